@@ -1,0 +1,225 @@
+// Host side of the C ABI: argument validation, the split heuristic and the launch
+// sequence. Validation and planning are pure host arithmetic (no HIP calls), so a
+// machine without a GPU can exercise them.
+#include <hip/hip_runtime_api.h>
+
+#include <algorithm>
+#include <cstdlib>
+
+#include "fta_internal.h"
+
+namespace fta {
+
+int mfma_rows_per_wg(int rows) { return rows > 128 ? 256 : 128; }
+
+namespace {
+
+inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+int esize(int dtype) { return dtype == FTA_F32 ? 4 : 2; }
+
+bool mfma_eligible(const fta_args& a, int rows) {
+  // The MFMA kernel takes row maxima before scaling, which needs a positive scale.
+  return (a.dtype == FTA_F16 || a.dtype == FTA_BF16) && (a.head_dim == 64 || a.head_dim == 128) && rows >= 16 &&
+         a.sm_scale > 0.f;
+}
+
+// Query heads that share both their cache head and their tree head.
+int heads_per_unit(const fta_args& a) {
+  const int g = a.num_q_heads / a.num_kv_heads;
+  return a.cur_heads == a.num_kv_heads ? g : 1;
+}
+
+int validate(const fta_args& a) {
+  if (!a.q || !a.k_cache || !a.v_cache || !a.cur_k || !a.cur_v || !a.mask || !a.kv_seq_len || !a.out)
+    return FTA_ERR_NULL_POINTER;
+  if (a.dtype != FTA_F32 && a.dtype != FTA_F16 && a.dtype != FTA_BF16) return FTA_ERR_DTYPE;
+  if (a.len_dtype != FTA_I32 && a.len_dtype != FTA_I64) return FTA_ERR_DTYPE;
+  if (a.head_dim != 32 && a.head_dim != 64 && a.head_dim != 128 && a.head_dim != 256) return FTA_ERR_HEAD_DIM;
+  if (a.cache_len != a.v_cache_len) return FTA_ERR_CACHE_LEN_MISMATCH;
+  if (a.block_size != 16 && a.block_size != 32 && a.block_size != 64 && a.block_size != 128)
+    return FTA_ERR_BLOCK_SIZE;
+  if (a.bsz <= 0 || a.num_q_heads <= 0 || a.num_kv_heads <= 0 || a.q_len <= 0 || a.cache_len < 0 ||
+      a.max_seq_len_hint < 0 || a.mid_splits < 0 || a.force_splits < 0)
+    return FTA_ERR_SHAPE;
+  if (a.num_q_heads % a.num_kv_heads != 0) return FTA_ERR_SHAPE;
+  if (a.cur_heads != a.num_kv_heads && a.cur_heads != a.num_q_heads) return FTA_ERR_SHAPE;
+  if (a.force_kernel < -1 || a.force_kernel > FTA_KERNEL_MFMA) return FTA_ERR_UNSUPPORTED;
+
+  // Rows are moved with 128-bit accesses: every row start must be 16-byte aligned.
+  const int vec = 16 / esize(a.dtype);
+  const int64_t* row_strides[] = {a.q_stride, a.k_stride, a.v_stride, a.ck_stride, a.cv_stride, a.out_stride};
+  for (const int64_t* s : row_strides)
+    for (int i = 0; i < 3; ++i) {
+      if (s[i] < 0) return FTA_ERR_STRIDE;
+      if (s[i] % vec != 0) return FTA_ERR_STRIDE;
+    }
+  const void* row_ptrs[] = {a.q, a.k_cache, a.v_cache, a.cur_k, a.cur_v, a.out};
+  for (const void* ptr : row_ptrs)
+    if (reinterpret_cast<uintptr_t>(ptr) % 16 != 0) return FTA_ERR_STRIDE;
+  for (int i = 0; i < 3; ++i)
+    if (a.mask_stride[i] < 0) return FTA_ERR_STRIDE;
+  return FTA_OK;
+}
+
+int plan(const fta_args& a, int num_cus, fta_plan_out* out) {
+  if (num_cus <= 0) num_cus = kDefaultCUs;
+  const int hpu = heads_per_unit(a);
+  const int rows = hpu * a.q_len;
+  const int units = a.num_q_heads / hpu;
+
+  int kernel = mfma_eligible(a, rows) ? FTA_KERNEL_MFMA : FTA_KERNEL_SHUFFLE;
+  if (a.force_kernel >= 0) {
+    if (a.force_kernel == FTA_KERNEL_MFMA && !mfma_eligible(a, rows)) return FTA_ERR_UNSUPPORTED;
+    kernel = a.force_kernel;
+  }
+  const int rows_per_wg = kernel == FTA_KERNEL_MFMA ? mfma_rows_per_wg(rows) : 16;
+  const int row_blocks = static_cast<int>(cdiv(rows, rows_per_wg));
+  // Workgroups one CU holds at a time (LDS- and register-bound, see the kernels).
+  const int wg_per_cu = kernel == FTA_KERNEL_MFMA ? (rows_per_wg == 256 ? 1 : 2) : 1;
+
+  const int64_t work_items = static_cast<int64_t>(a.bsz) * units * row_blocks;
+  const int64_t t_cap = a.max_seq_len_hint > 0 ? std::min(a.max_seq_len_hint, a.cache_len) : a.cache_len;
+  const int gran = std::max(a.block_size, kKeyTile);
+
+  // A split costs one fp32 partial written by stage 1 and read back by stage 2; in
+  // units of "keys of K/V traffic" that is 2*rows*D*4 / (2*D*esize) keys.
+  const int64_t partial_keys = 4LL * std::min(rows, rows_per_wg) / esize(a.dtype);
+  const int64_t min_chunk_fill = std::max<int64_t>(gran, 4 * kKeyTile);          // when CUs would idle otherwise
+  const int64_t min_chunk_over = std::max<int64_t>(min_chunk_fill, 8 * partial_keys);  // when only balancing
+
+  const int64_t target = static_cast<int64_t>(num_cus) * wg_per_cu;
+  int64_t s_fill = cdiv(target, work_items);
+  s_fill = std::min(s_fill, std::max<int64_t>(1, t_cap / min_chunk_fill));
+  // Ragged batches: lengths are not known on the host, so oversubscribe the CUs
+  // with equal-sized chunks; a single sequence has nothing to balance.
+  int64_t s_over = 1;
+  if (a.bsz > 1) {
+    s_over = cdiv(8 * target, work_items);
+    s_over = std::min(s_over, std::max<int64_t>(1, t_cap / min_chunk_over));
+  }
+  int64_t splits = std::max<int64_t>(1, std::max(s_fill, s_over));
+  if (a.force_splits > 0) splits = a.force_splits;
+  if (const char* env = std::getenv("FTA_FORCE_SPLITS")) {
+    const int v = std::atoi(env);
+    if (v > 0) splits = v;
+  }
+  // Never more splits than blocks of the reference granularity, so that a scratch
+  // buffer sized like the reference's (flash_tree_attn.py:274-281) always fits.
+  splits = std::min<int64_t>(splits, std::max<int64_t>(1, cdiv(t_cap, gran)));
+  int64_t chunk = cdiv(cdiv(std::max<int64_t>(t_cap, 1), splits), gran) * gran;
+  splits = std::max<int64_t>(1, cdiv(std::max<int64_t>(t_cap, 1), chunk));
+
+  out->kernel = kernel;
+  out->num_splits = static_cast<int32_t>(splits);
+  out->chunk = static_cast<int32_t>(chunk);
+  out->rows_per_group = rows;
+  out->rows_per_wg = rows_per_wg;
+  out->row_blocks = row_blocks;
+  out->num_workgroups = static_cast<int32_t>(work_items * splits);
+  out->reserved = 0;
+  out->mid_lse_elems = splits > 1 ? static_cast<int64_t>(a.bsz) * a.num_q_heads * splits * a.q_len : 0;
+  out->mid_o_elems = out->mid_lse_elems * a.head_dim;
+  return FTA_OK;
+}
+
+}  // namespace
+}  // namespace fta
+
+extern "C" {
+
+int fta_abi_version(void) { return FTA_ABI_VERSION; }
+
+const char* fta_strerror(int status) {
+  switch (status) {
+    case FTA_OK: return "ok";
+    case FTA_ERR_NULL_POINTER: return "a required pointer is NULL";
+    case FTA_ERR_HEAD_DIM: return "head_dim must be one of 32, 64, 128, 256";
+    case FTA_ERR_BLOCK_SIZE: return "block_size must be one of 16, 32, 64, 128";
+    case FTA_ERR_CACHE_LEN_MISMATCH: return "k_cache and v_cache have different sequence lengths";
+    case FTA_ERR_SCRATCH_TOO_SMALL: return "mid_output / mid_output_lse hold fewer splits than the plan needs";
+    case FTA_ERR_DTYPE: return "unsupported dtype";
+    case FTA_ERR_SHAPE: return "inconsistent shapes";
+    case FTA_ERR_STRIDE: return "unsupported strides: inner stride must be 1 and rows 16-byte aligned";
+    case FTA_ERR_UNSUPPORTED: return "no kernel instantiated for this combination";
+    case FTA_ERR_LAUNCH: return "HIP kernel launch failed";
+    case FTA_ERR_NO_DEVICE: return "no HIP device available";
+    default: return "unknown fta status";
+  }
+}
+
+int fta_validate(const fta_args* args) {
+  if (!args) return FTA_ERR_NULL_POINTER;
+  return fta::validate(*args);
+}
+
+int fta_plan(const fta_args* args, int num_cus, fta_plan_out* plan) {
+  if (!args || !plan) return FTA_ERR_NULL_POINTER;
+  // Planning needs consistent sizes but no pointers.
+  fta_args a = *args;
+  // 16-byte aligned stand-in so that validate() only judges the sizes.
+  alignas(16) static const char aligned_dummy[16] = {0};
+  const void* d = aligned_dummy;
+  a.q = a.k_cache = a.v_cache = a.cur_k = a.cur_v = a.kv_seq_len = d;
+  a.mask = reinterpret_cast<const float*>(d);
+  a.out = const_cast<void*>(d);
+  if (int st = fta::validate(a)) return st;
+  return fta::plan(a, num_cus, plan);
+}
+
+int fta_device_cus(void) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return FTA_ERR_NO_DEVICE;
+  int cus = 0;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return FTA_ERR_NO_DEVICE;
+  return cus;
+}
+
+int fta_decode(const fta_args* args, void* hip_stream) {
+  if (!args) return FTA_ERR_NULL_POINTER;
+  const fta_args& a = *args;
+  if (int st = fta::validate(a)) return st;
+  static thread_local int cached_cus = 0;
+  if (cached_cus <= 0) {
+    cached_cus = fta_device_cus();
+    if (cached_cus <= 0) return FTA_ERR_NO_DEVICE;
+  }
+  fta_plan_out pl;
+  if (int st = fta::plan(a, cached_cus, &pl)) return st;
+  if (pl.num_splits > 1) {
+    if (!a.mid_o || !a.mid_lse) return FTA_ERR_NULL_POINTER;
+    if (a.mid_splits < pl.num_splits) return FTA_ERR_SCRATCH_TOO_SMALL;
+    for (int i = 0; i < 4; ++i)
+      if (a.mid_o_stride[i] < 0 || a.mid_o_stride[i] % 4 != 0) return FTA_ERR_STRIDE;
+    for (int i = 0; i < 3; ++i)
+      if (a.mid_lse_stride[i] < 0) return FTA_ERR_STRIDE;
+    if (reinterpret_cast<uintptr_t>(a.mid_o) % 16 != 0) return FTA_ERR_STRIDE;
+  }
+
+  fta::KernelParams p{};
+  p.q = a.q; p.k = a.k_cache; p.v = a.v_cache; p.ck = a.cur_k; p.cv = a.cur_v;
+  p.mask = a.mask; p.lens = a.kv_seq_len; p.out = a.out; p.mid_o = a.mid_o; p.mid_lse = a.mid_lse;
+  p.bsz = a.bsz; p.num_q_heads = a.num_q_heads; p.q_len = a.q_len; p.cache_len = a.cache_len;
+  p.chunk = pl.chunk; p.num_splits = pl.num_splits;
+  p.heads_per_unit = pl.rows_per_group / a.q_len;
+  p.units = a.num_q_heads / p.heads_per_unit;
+  p.kv_group = a.num_q_heads / a.num_kv_heads;
+  p.cur_group = a.num_q_heads / a.cur_heads;
+  p.rows = pl.rows_per_group; p.rows_per_wg = pl.rows_per_wg; p.row_blocks = pl.row_blocks;
+  p.len_is_i64 = a.len_dtype == FTA_I64;
+  p.scale_log2 = a.sm_scale * fta::kLog2e;
+  for (int i = 0; i < 3; ++i) {
+    p.q_stride[i] = a.q_stride[i]; p.k_stride[i] = a.k_stride[i]; p.v_stride[i] = a.v_stride[i];
+    p.ck_stride[i] = a.ck_stride[i]; p.cv_stride[i] = a.cv_stride[i]; p.mask_stride[i] = a.mask_stride[i];
+    p.out_stride[i] = a.out_stride[i]; p.mid_lse_stride[i] = a.mid_lse_stride[i];
+  }
+  for (int i = 0; i < 4; ++i) p.mid_o_stride[i] = a.mid_o_stride[i];
+
+  int st = pl.kernel == FTA_KERNEL_MFMA ? fta::launch_stage1_mfma(p, a.dtype, a.head_dim, hip_stream)
+                                        : fta::launch_stage1_shuffle(p, a.dtype, a.head_dim, hip_stream);
+  if (st) return st;
+  if (pl.num_splits > 1) st = fta::launch_stage2_merge(p, a.dtype, a.head_dim, hip_stream);
+  return st;
+}
+
+}  // extern "C"

@@ -1,0 +1,63 @@
+// Internal declarations shared by the host side and the HIP kernels.
+#pragma once
+#include <stdint.h>
+#include "fta.h"
+
+namespace fta {
+
+constexpr int kKeyTile = 64;        // keys per LDS tile in every stage-1 kernel
+constexpr int kDefaultCUs = 256;    // MI355X: 8 XCDs x 32 CUs
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// Kernel-side view of one call. A "unit" is a set of `heads_per_unit` consecutive
+// query heads that read the same cache head AND the same tree head, so one K/V
+// stream serves rows = heads_per_unit * q_len query rows.
+struct KernelParams {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* ck;
+  const void* cv;
+  const float* mask;
+  const void* lens;
+  void* out;
+  float* mid_o;
+  float* mid_lse;
+
+  int32_t bsz;
+  int32_t num_q_heads;
+  int32_t q_len;
+  int32_t cache_len;
+  int32_t chunk;
+  int32_t num_splits;
+  int32_t heads_per_unit;
+  int32_t units;          // num_q_heads / heads_per_unit
+  int32_t kv_group;       // query heads per cache head
+  int32_t cur_group;      // query heads per tree head
+  int32_t rows;           // heads_per_unit * q_len
+  int32_t rows_per_wg;
+  int32_t row_blocks;
+  int32_t len_is_i64;
+  float scale_log2;       // sm_scale * log2(e)
+
+  int64_t q_stride[3];
+  int64_t k_stride[3];
+  int64_t v_stride[3];
+  int64_t ck_stride[3];
+  int64_t cv_stride[3];
+  int64_t mask_stride[3];
+  int64_t out_stride[3];
+  int64_t mid_o_stride[4];
+  int64_t mid_lse_stride[3];
+};
+
+// Launchers implemented in the .hip files. Each returns a fta_status.
+int launch_stage1_shuffle(const KernelParams& p, int dtype, int head_dim, void* stream);
+int launch_stage1_mfma(const KernelParams& p, int dtype, int head_dim, void* stream);
+int launch_stage2_merge(const KernelParams& p, int dtype, int head_dim, void* stream);
+
+// Rows one MFMA workgroup holds for a unit of `rows` query rows (host + device agree on it).
+int mfma_rows_per_wg(int rows);
+
+}  // namespace fta

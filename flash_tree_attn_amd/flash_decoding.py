@@ -1,0 +1,213 @@
+"""`flash_decoding_attention`: drop-in for the reference function of the same name
+(flash_tree_attn.py:216-376), running hand-written gfx950 kernels through the C ABI
+of libfta.so. PyTorch is used for device memory and the current stream only.
+
+Differences from the reference that a caller can observe (all deliberate):
+* `output=`, when given, receives the FINAL result and is returned; the reference
+  leaves the cache-only attention there and returns a new tensor
+  (flash_tree_attn.py:373-376).
+* `mid_output` / `mid_output_lse` are scratch for at most `plan.num_splits` splits
+  (never more than ceil(max_len / block_size), so reference-sized buffers fit).
+* No host sync: `kv_seq_len.max().item()` (flash_tree_attn.py:272) is not needed;
+  `max_seq_len_in_batch` is only a hint that shrinks the grid.
+* fp16, bf16 and fp32 inputs; `current_k/current_v` with num_kv_heads or num_heads
+  heads; any q_len >= 1; `mask` float (additive, flash_tree_attn.py:368) or bool.
+* A query row whose every logit is -inf yields zeros (the reference yields NaN).
+There is no CPU or eager fallback: CPU tensors and a missing library raise.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+_DTYPES = {torch.float32: _lib.FTA_F32, torch.float16: _lib.FTA_F16, torch.bfloat16: _lib.FTA_BF16}
+
+
+class FtaAssertionError(ValueError, AssertionError):
+    """Raised where the reference trips a bare `assert` (flash_tree_attn.py:263-291)."""
+
+
+_ASSERT_STATUSES = {-2, -3, -4, -5}
+_cu_count = {}
+
+
+def _check(status: int) -> None:
+    if status == 0:
+        return
+    text = _lib.load().fta_strerror(status).decode()
+    if status in _ASSERT_STATUSES:
+        raise FtaAssertionError(f"fta status {status}: {text}")
+    _lib.check(status)
+
+
+def _rows_ok(t: torch.Tensor) -> bool:
+    vec = 16 // t.element_size()
+    return (t.stride(-1) == 1 and all(s % vec == 0 and s >= 0 for s in t.stride()[:-1])
+            and t.data_ptr() % 16 == 0)
+
+
+def _as_rows(t: torch.Tensor) -> torch.Tensor:
+    """128-bit row access needs unit inner stride and 16-byte aligned rows; anything
+    else is copied once (the reference honours arbitrary strides, flash_tree_attn.py:311-330)."""
+    return t if _rows_ok(t) else t.contiguous()
+
+
+def _num_cus(device: torch.device) -> int:
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    if idx not in _cu_count:
+        _cu_count[idx] = torch.cuda.get_device_properties(idx).multi_processor_count
+    return _cu_count[idx]
+
+
+def _prepare_mask(mask: torch.Tensor, bsz: int, hq: int, L: int, device) -> torch.Tensor:
+    if mask.device != device:
+        raise ValueError("mask must live on the same device as q")
+    if mask.dtype == torch.bool:
+        m = torch.zeros(mask.shape, dtype=torch.float32, device=device)
+        m.masked_fill_(~mask, float("-inf"))
+        mask = m
+    elif mask.dtype != torch.float32:
+        mask = mask.float()
+    if mask.dim() > 4 or mask.dim() < 2:
+        raise ValueError(f"mask must be [q_len, q_len] up to [bsz, num_heads, q_len, q_len], got {tuple(mask.shape)}")
+    while mask.dim() < 4:
+        mask = mask.unsqueeze(0)
+    try:
+        mask = mask.expand(bsz, hq, L, L)
+    except RuntimeError as e:
+        raise ValueError(f"mask of shape {tuple(mask.shape)} does not broadcast to {(bsz, hq, L, L)}") from e
+    if mask.stride(3) != 1 and L > 1:
+        mask = mask.contiguous()
+    return mask
+
+
+def build_args(q, k_cache, v_cache, current_k, current_v, mask, kv_seq_len, block_size,
+               max_seq_len_in_batch, sm_scale, kv_group_num, force_splits=0, force_kernel=-1):
+    """Validates tensors on the Python side and fills an FtaArgs (without out/scratch).
+    Returns (args, keepalive) where keepalive holds every tensor the pointers refer to."""
+    if q.dim() != 4:
+        raise ValueError(f"q must be [bsz, num_heads, q_len, head_dim], got {tuple(q.shape)}")
+    bsz, hq, L, D = q.shape
+    dev = q.device
+    if dev.type != "cuda":
+        raise RuntimeError("flash_decoding_attention runs on the GPU only; there is no CPU fallback")
+    if q.dtype not in _DTYPES:
+        raise ValueError(f"unsupported dtype {q.dtype}")
+    for name, t in (("k_cache", k_cache), ("v_cache", v_cache), ("current_k", current_k), ("current_v", current_v)):
+        if t.dim() != 4:
+            raise ValueError(f"{name} must be 4-dimensional, got {tuple(t.shape)}")
+        if t.dtype != q.dtype or t.device != dev:
+            raise ValueError(f"{name} must have q's dtype and device")
+        if t.size(0) != bsz or t.size(3) != D:
+            raise ValueError(f"{name} has shape {tuple(t.shape)}, incompatible with q {tuple(q.shape)}")
+    hkv = k_cache.size(1)
+    if v_cache.size(1) != hkv or hkv * int(kv_group_num) != hq:
+        raise ValueError(f"num_heads {hq} != num_kv_heads {hkv} * kv_group_num {kv_group_num}")
+    if current_k.shape != current_v.shape or current_k.size(2) != L:
+        raise ValueError("current_k/current_v must be [bsz, num_kv_heads (or num_heads), q_len, head_dim]")
+    if kv_seq_len.device != dev or kv_seq_len.dtype not in (torch.int32, torch.int64) or kv_seq_len.numel() != bsz:
+        raise ValueError("kv_seq_len must be an int32/int64 tensor of bsz elements on q's device")
+
+    q, k_cache, v_cache = _as_rows(q), _as_rows(k_cache), _as_rows(v_cache)
+    current_k, current_v = _as_rows(current_k), _as_rows(current_v)
+    kv_seq_len = kv_seq_len.contiguous().view(-1)
+    mask = _prepare_mask(mask, bsz, hq, L, dev)
+
+    a = _lib.FtaArgs()
+    a.q, a.k_cache, a.v_cache = q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr()
+    a.cur_k, a.cur_v = current_k.data_ptr(), current_v.data_ptr()
+    a.mask, a.kv_seq_len = mask.data_ptr(), kv_seq_len.data_ptr()
+    a.bsz, a.num_q_heads, a.num_kv_heads, a.cur_heads = bsz, hq, hkv, current_k.size(1)
+    a.q_len, a.head_dim = L, D
+    a.cache_len, a.v_cache_len = k_cache.size(2), v_cache.size(2)
+    a.block_size = int(block_size)
+    a.max_seq_len_hint = 0 if max_seq_len_in_batch is None else max(int(max_seq_len_in_batch), 1)
+    a.dtype = _DTYPES[q.dtype]
+    a.len_dtype = _lib.FTA_I64 if kv_seq_len.dtype == torch.int64 else _lib.FTA_I32
+    a.force_splits, a.force_kernel = int(force_splits), int(force_kernel)
+    a.sm_scale = float(1.0 / (D ** 0.5) if sm_scale is None else sm_scale)
+    a.q_stride[:] = q.stride()[:3]
+    a.k_stride[:] = k_cache.stride()[:3]
+    a.v_stride[:] = v_cache.stride()[:3]
+    a.ck_stride[:] = current_k.stride()[:3]
+    a.cv_stride[:] = current_v.stride()[:3]
+    a.mask_stride[:] = mask.stride()[:3]
+    return a, (q, k_cache, v_cache, current_k, current_v, mask, kv_seq_len)
+
+
+def plan_for(args: "_lib.FtaArgs", num_cus: int) -> "_lib.FtaPlanOut":
+    pl = _lib.FtaPlanOut()
+    _check(_lib.load().fta_plan(C.byref(args), int(num_cus), C.byref(pl)))
+    return pl
+
+
+def flash_decoding_attention(
+    q: torch.Tensor,
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    current_k: torch.Tensor,
+    current_v: torch.Tensor,
+    mask: torch.Tensor,
+    kv_seq_len: torch.Tensor,
+    block_size: int = 64,
+    max_seq_len_in_batch: Optional[int] = None,
+    output: Optional[torch.Tensor] = None,
+    mid_output: Optional[torch.Tensor] = None,
+    mid_output_lse: Optional[torch.Tensor] = None,
+    sm_scale: Optional[float] = None,
+    kv_group_num: int = 1,
+    *,
+    _force_splits: int = 0,
+    _force_kernel: int = -1,
+) -> torch.Tensor:
+    """Tree-attention decode (speculative-decoding verification).
+
+    Same parameters, order and defaults as the reference (flash_tree_attn.py:216-231):
+      q [bsz, num_heads, q_len, head_dim]; k_cache / v_cache [bsz, num_kv_heads, ctx, head_dim];
+      current_k / current_v [bsz, num_kv_heads, q_len, head_dim]; mask [q_len, q_len] or
+      [bsz, num_heads, q_len, q_len], ADDED to the tree logits; kv_seq_len [bsz].
+    Returns [bsz, num_heads, q_len, head_dim] in q's dtype.
+    """
+    lib = _lib.load()
+    args, keep = build_args(q, k_cache, v_cache, current_k, current_v, mask, kv_seq_len, block_size,
+                            max_seq_len_in_batch, sm_scale, kv_group_num, _force_splits, _force_kernel)
+    bsz, hq, L, D = q.shape
+    dev = q.device
+    pl = plan_for(args, _num_cus(dev))
+
+    if output is None:
+        output = torch.empty((bsz, hq, L, D), dtype=q.dtype, device=dev)
+    else:
+        if output.shape != (bsz, hq, L, D) or output.dtype != q.dtype or output.device != dev:
+            raise FtaAssertionError("output must be [bsz, num_heads, q_len, head_dim] with q's dtype and device")
+        if not _rows_ok(output):
+            raise ValueError("output needs unit inner stride and 16-byte aligned rows")
+    args.out = output.data_ptr()
+    args.out_stride[:] = output.stride()[:3]
+
+    if pl.num_splits > 1:
+        if mid_output is None:
+            mid_output = torch.empty((bsz, hq, pl.num_splits, L, D), dtype=torch.float32, device=dev)
+        if mid_output_lse is None:
+            mid_output_lse = torch.empty((bsz, hq, pl.num_splits, L), dtype=torch.float32, device=dev)
+        for name, t, nd in (("mid_output", mid_output, 5), ("mid_output_lse", mid_output_lse, 4)):
+            if t.dim() != nd or t.dtype != torch.float32 or t.device != dev or t.stride(-1) != 1:
+                raise FtaAssertionError(f"{name} must be a float32 tensor with {nd} dims on q's device")
+            if t.size(0) < bsz or t.size(1) != hq or t.size(3) != L:
+                raise FtaAssertionError(f"{name} has incompatible shape {tuple(t.shape)}")
+        if mid_output.size(4) != D:
+            raise FtaAssertionError(f"mid_output has incompatible shape {tuple(mid_output.shape)}")
+        args.mid_o, args.mid_lse = mid_output.data_ptr(), mid_output_lse.data_ptr()
+        args.mid_splits = min(mid_output.size(2), mid_output_lse.size(2))
+        args.mid_o_stride[:] = mid_output.stride()[:4]
+        args.mid_lse_stride[:] = mid_output_lse.stride()[:3]
+
+    with torch.cuda.device(dev):
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        _check(lib.fta_decode(C.byref(args), C.c_void_p(stream)))
+    del keep
+    return output

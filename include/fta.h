@@ -1,0 +1,146 @@
+/*
+ * fta.h - C ABI of the MI355X (gfx950) tree-attention decode library.
+ *
+ * The reference exposes this path as one Python function,
+ *   flash_decoding_attention(q, k_cache, v_cache, current_k, current_v, mask,
+ *                            kv_seq_len, block_size, max_seq_len_in_batch,
+ *                            output, mid_output, mid_output_lse, sm_scale,
+ *                            kv_group_num)            (flash_tree_attn.py:216-231)
+ * which launches two Triton kernels and a dozen eager ops. This header is what a
+ * binding for that function talks to: plain pointers, sizes and element strides,
+ * no torch types. Every function returns 0 (FTA_OK) or a negative fta_status and
+ * never throws, allocates device memory, or synchronises the device.
+ */
+#ifndef FTA_H_
+#define FTA_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FTA_ABI_VERSION 1
+
+typedef enum fta_status {
+  FTA_OK = 0,
+  FTA_ERR_NULL_POINTER = -1,      /* a required pointer is NULL */
+  FTA_ERR_HEAD_DIM = -2,          /* head_dim not in {32,64,128,256}   (flash_tree_attn.py:263) */
+  FTA_ERR_BLOCK_SIZE = -3,        /* block_size not in {16,32,64,128}  (flash_tree_attn.py:268) */
+  FTA_ERR_CACHE_LEN_MISMATCH = -4,/* k_cache/v_cache lengths differ    (flash_tree_attn.py:264) */
+  FTA_ERR_SCRATCH_TOO_SMALL = -5, /* mid_o/mid_lse hold fewer splits than planned (flash_tree_attn.py:286-291) */
+  FTA_ERR_DTYPE = -6,             /* unknown dtype / length dtype enum */
+  FTA_ERR_SHAPE = -7,             /* non-positive size, Hq != Hkv*G, current_k heads not Hkv or Hq */
+  FTA_ERR_STRIDE = -8,            /* negative stride, or rows not 16-byte aligned for the vector path */
+  FTA_ERR_UNSUPPORTED = -9,       /* combination no kernel is instantiated for */
+  FTA_ERR_LAUNCH = -10,           /* HIP reported a launch error */
+  FTA_ERR_NO_DEVICE = -11         /* no gfx950 device is visible to HIP */
+} fta_status;
+
+typedef enum fta_dtype { FTA_F32 = 0, FTA_F16 = 1, FTA_BF16 = 2 } fta_dtype;
+typedef enum fta_len_dtype { FTA_I32 = 0, FTA_I64 = 1 } fta_len_dtype;
+
+/* Which stage-1 kernel a plan selects. */
+typedef enum fta_kernel {
+  FTA_KERNEL_SHUFFLE = 0,  /* wavefront-shuffle reductions: any dtype / head_dim / q_len */
+  FTA_KERNEL_MFMA = 1      /* MFMA tiles: f16/bf16, head_dim 64/128, group rows >= 16 */
+} fta_kernel;
+
+/*
+ * One call of the path. All strides are in ELEMENTS of the tensor they index;
+ * the innermost (head_dim, and mask column) stride must be 1.
+ * Shapes (reference docstring, flash_tree_attn.py:235-246):
+ *   q         [bsz, num_q_heads, q_len, head_dim]
+ *   k_cache   [bsz, num_kv_heads, cache_len, head_dim]   (same for v_cache)
+ *   cur_k     [bsz, cur_heads, q_len, head_dim]          cur_heads = num_kv_heads or num_q_heads
+ *   mask      float32, additive (flash_tree_attn.py:368); strides may be 0 to broadcast
+ *             over batch and/or head, i.e. [q_len,q_len] .. [bsz,num_q_heads,q_len,q_len]
+ *   kv_seq_len[bsz] int32 or int64 (flash_tree_attn.py:434 passes int64)
+ *   out       [bsz, num_q_heads, q_len, head_dim], dtype of q: the FINAL result
+ *   mid_o     float32 [bsz, num_q_heads, mid_splits, q_len, head_dim]  (flash_tree_attn.py:276-279)
+ *   mid_lse   float32 [bsz, num_q_heads, mid_splits, q_len]            (flash_tree_attn.py:280-281)
+ * mid_o / mid_lse are scratch; they may be NULL when the plan has num_splits == 1.
+ */
+typedef struct fta_args {
+  const void* q;
+  const void* k_cache;
+  const void* v_cache;
+  const void* cur_k;
+  const void* cur_v;
+  const float* mask;
+  const void* kv_seq_len;
+  void* out;
+  float* mid_o;
+  float* mid_lse;
+
+  int32_t bsz;
+  int32_t num_q_heads;
+  int32_t num_kv_heads;
+  int32_t cur_heads;
+  int32_t q_len;
+  int32_t head_dim;
+  int32_t cache_len;        /* k_cache.size(2) */
+  int32_t v_cache_len;      /* v_cache.size(2), must equal cache_len */
+  int32_t block_size;       /* the reference's split granularity (flash_tree_attn.py:268) */
+  int32_t max_seq_len_hint; /* max_seq_len_in_batch, or 0 when the caller gave none */
+  int32_t mid_splits;       /* size(2) of mid_o / mid_lse, 0 when they are NULL */
+  int32_t dtype;            /* fta_dtype of q/k/v/cur/out */
+  int32_t len_dtype;        /* fta_len_dtype of kv_seq_len */
+  int32_t force_splits;     /* 0 = heuristic; >0 pins the split count (tuning, tests) */
+  int32_t force_kernel;     /* -1 = heuristic; else an fta_kernel */
+  float sm_scale;
+
+  int64_t q_stride[3];      /* batch, head, row */
+  int64_t k_stride[3];      /* batch, head, position */
+  int64_t v_stride[3];
+  int64_t ck_stride[3];     /* batch, head, row */
+  int64_t cv_stride[3];
+  int64_t mask_stride[3];   /* batch, head, row (column stride is 1) */
+  int64_t out_stride[3];    /* batch, head, row */
+  int64_t mid_o_stride[4];  /* batch, head, split, row */
+  int64_t mid_lse_stride[3];/* batch, head, split */
+} fta_args;
+
+/* What the split heuristic decided for one fta_args (pure host arithmetic). */
+typedef struct fta_plan_out {
+  int32_t kernel;         /* fta_kernel */
+  int32_t num_splits;     /* grid extent along the KV sequence; 1 = single pass, no scratch, no stage 2 */
+  int32_t chunk;          /* keys per split; a multiple of block_size and of the kernel's key tile */
+  int32_t rows_per_group; /* kv_group_num * q_len: query rows that share one K/V stream */
+  int32_t rows_per_wg;    /* query rows one workgroup holds */
+  int32_t row_blocks;     /* ceil(rows_per_group / rows_per_wg) */
+  int32_t num_workgroups; /* stage-1 grid size */
+  int32_t reserved;
+  int64_t mid_o_elems;    /* float32 elements a dense mid_o for this plan needs */
+  int64_t mid_lse_elems;
+} fta_plan_out;
+
+/* ABI version of the loaded library (== FTA_ABI_VERSION it was built with). */
+int fta_abi_version(void);
+
+/* Static, human-readable text for a status code. */
+const char* fta_strerror(int status);
+
+/* Argument checks of flash_tree_attn.py:263-268,286-291 plus the stride/dtype
+ * contract of this library. Pure host code: callable without a GPU; pointers are
+ * only compared against NULL, never dereferenced. */
+int fta_validate(const fta_args* args);
+
+/* The split-count heuristic that replaces "one split per block_size keys"
+ * (flash_tree_attn.py:266-274, :293-299). Pure host code. `num_cus` is the number
+ * of compute units to fill (256 on MI355X); pass 0 to use that default. Does not
+ * look at kv_seq_len values (no host sync, unlike flash_tree_attn.py:272). */
+int fta_plan(const fta_args* args, int num_cus, fta_plan_out* plan);
+
+/* Runs the whole path (stage 1 with the tree block folded in, then the LSE merge
+ * when the plan has more than one split) on `hip_stream` (a hipStream_t; NULL is
+ * the default stream). Replaces flash_tree_attn.py:293-376. Asynchronous. */
+int fta_decode(const fta_args* args, void* hip_stream);
+
+/* Number of compute units of the current HIP device, or a negative fta_status. */
+int fta_device_cus(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FTA_H_ */

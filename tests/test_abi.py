@@ -1,0 +1,178 @@
+"""CPU-only checks of the C-ABI library: it loads, exports every symbol include/fta.h
+declares, validates arguments like the reference's asserts (flash_tree_attn.py:263-291)
+and plans splits sensibly. No kernel is launched here."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from flash_tree_attn_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def base_args(**kw):
+    a = _lib.FtaArgs()
+    ptr = 0x1000  # never dereferenced by validate/plan
+    for f in ("q", "k_cache", "v_cache", "cur_k", "cur_v", "mask", "kv_seq_len", "out"):
+        setattr(a, f, ptr)
+    cfg = dict(bsz=8, num_q_heads=32, num_kv_heads=8, cur_heads=8, q_len=64, head_dim=128, cache_len=8192,
+               v_cache_len=8192, block_size=64, max_seq_len_hint=0, mid_splits=0, dtype=_lib.FTA_BF16,
+               len_dtype=_lib.FTA_I64, force_splits=0, force_kernel=-1, sm_scale=128 ** -0.5)
+    cfg.update(kw)
+    for k, v in cfg.items():
+        setattr(a, k, v)
+    D, L, T = a.head_dim, a.q_len, a.cache_len
+    a.q_stride[:] = [a.num_q_heads * L * D, L * D, D]
+    a.k_stride[:] = [a.num_kv_heads * T * D, T * D, D]
+    a.v_stride[:] = a.k_stride[:]
+    a.ck_stride[:] = [a.cur_heads * L * D, L * D, D]
+    a.cv_stride[:] = a.ck_stride[:]
+    a.mask_stride[:] = [0, 0, L]
+    a.out_stride[:] = a.q_stride[:]
+    return a
+
+
+def plan(fta_lib, a, cus=256):
+    pl = _lib.FtaPlanOut()
+    st = fta_lib.fta_plan(C.byref(a), cus, C.byref(pl))
+    return st, pl
+
+
+def test_header_symbols_exported(fta_lib):
+    header = open(os.path.join(ROOT, "include", "fta.h")).read()
+    declared = set(re.findall(r"^\s*(?:int|const char\*)\s+(fta_\w+)\s*\(", header, flags=re.M))
+    assert declared == set(_lib.EXPORTED_SYMBOLS)
+    for name in declared:
+        assert hasattr(fta_lib, name), name
+    assert fta_lib.fta_abi_version() == _lib.ABI_VERSION
+    assert int(re.search(r"#define FTA_ABI_VERSION (\d+)", header).group(1)) == _lib.ABI_VERSION
+
+
+def test_struct_layout_matches_header(fta_lib):
+    # 10 pointers, 15 int32 + 1 float, 9 stride arrays (8 of 3 + 1 of 4 int64)
+    assert C.sizeof(_lib.FtaArgs) == 10 * 8 + 16 * 4 + (8 * 3 + 4) * 8
+    assert C.sizeof(_lib.FtaPlanOut) == 8 * 4 + 2 * 8
+
+
+def test_strerror(fta_lib):
+    assert fta_lib.fta_strerror(0) == b"ok"
+    seen = set()
+    for st in range(-11, 0):
+        s = fta_lib.fta_strerror(st)
+        assert s and s != b"unknown fta status"
+        seen.add(s)
+    assert len(seen) == 11
+    assert fta_lib.fta_strerror(-99) == b"unknown fta status"
+
+
+@pytest.mark.parametrize("kw, status", [
+    (dict(head_dim=96), -2), (dict(head_dim=512), -2),          # flash_tree_attn.py:263
+    (dict(block_size=48), -3), (dict(block_size=256), -3),      # flash_tree_attn.py:268
+    (dict(v_cache_len=4096), -4),                               # flash_tree_attn.py:264
+    (dict(dtype=7), -6), (dict(len_dtype=3), -6),
+    (dict(bsz=0), -7), (dict(num_q_heads=30), -7), (dict(cur_heads=16), -7), (dict(q_len=0), -7),
+    (dict(force_kernel=5), -9),
+])
+def test_validate_rejects(fta_lib, kw, status):
+    a = base_args(**kw)
+    assert fta_lib.fta_validate(C.byref(a)) == status
+    assert plan(fta_lib, a)[0] == status
+
+
+def test_validate_pointer_and_stride_rules(fta_lib):
+    a = base_args()
+    assert fta_lib.fta_validate(C.byref(a)) == 0
+    assert fta_lib.fta_validate(None) == -1
+    a.mask = None
+    assert fta_lib.fta_validate(C.byref(a)) == -1
+    a = base_args()
+    a.k_stride[2] = 130  # rows no longer 16-byte aligned
+    assert fta_lib.fta_validate(C.byref(a)) == -8
+    a = base_args()
+    a.q = 0x1004
+    assert fta_lib.fta_validate(C.byref(a)) == -8
+    a = base_args()
+    a.v_stride[0] = -1
+    assert fta_lib.fta_validate(C.byref(a)) == -8
+
+
+def test_decode_without_scratch_or_device_fails_cleanly(fta_lib):
+    """fta_decode validates before touching HIP; on a GPU-less host it must return an
+    error status instead of crashing."""
+    a = base_args(head_dim=96)
+    assert fta_lib.fta_decode(C.byref(a), None) == -2
+    import torch
+    if not torch.cuda.is_available():
+        a = base_args()
+        assert fta_lib.fta_decode(C.byref(a), None) == -11
+
+
+CASES = [
+    dict(),                                                                                     # config 3
+    dict(bsz=4, num_q_heads=32, num_kv_heads=32, cur_heads=32, q_len=26, cache_len=4096, v_cache_len=4096, dtype=_lib.FTA_F16),
+    dict(bsz=1, cache_len=131072, v_cache_len=131072),                                          # config 4
+    dict(bsz=64, num_q_heads=64, q_len=16, cache_len=32768, v_cache_len=32768),                 # config 5
+    dict(bsz=1, num_q_heads=8, num_kv_heads=8, cur_heads=8, q_len=4, head_dim=64, cache_len=256, v_cache_len=256, dtype=_lib.FTA_F32),
+    dict(bsz=2, cache_len=0, v_cache_len=0),
+    dict(bsz=3, cache_len=100, v_cache_len=100, block_size=16),
+    dict(bsz=2, cache_len=100000, v_cache_len=100000, block_size=128, max_seq_len_hint=777),
+]
+
+
+@pytest.mark.parametrize("kw", CASES)
+@pytest.mark.parametrize("cus", [256, 64, 1])
+def test_plan_properties(fta_lib, kw, cus):
+    a = base_args(**kw)
+    st, pl = plan(fta_lib, a, cus)
+    assert st == 0
+    t_cap = min(a.max_seq_len_hint, a.cache_len) if a.max_seq_len_hint else a.cache_len
+    gran = max(a.block_size, 64)
+    assert pl.num_splits >= 1
+    assert pl.chunk % a.block_size == 0 and pl.chunk % 64 == 0 and pl.chunk >= gran
+    # the splits cover every key exactly once ...
+    assert pl.num_splits * pl.chunk >= t_cap
+    assert (pl.num_splits - 1) * pl.chunk < max(t_cap, 1)
+    # ... and never outnumber the reference's block count, so its scratch shapes fit
+    assert pl.num_splits <= max(1, -(-t_cap // a.block_size))
+    hpu = a.num_q_heads // a.num_kv_heads if a.cur_heads == a.num_kv_heads else 1
+    assert pl.rows_per_group == hpu * a.q_len
+    assert pl.row_blocks == -(-pl.rows_per_group // pl.rows_per_wg)
+    assert pl.num_workgroups == a.bsz * (a.num_q_heads // hpu) * pl.row_blocks * pl.num_splits
+    if pl.num_splits > 1:
+        assert pl.mid_lse_elems == a.bsz * a.num_q_heads * pl.num_splits * a.q_len
+        assert pl.mid_o_elems == pl.mid_lse_elems * a.head_dim
+    else:
+        assert pl.mid_o_elems == 0 and pl.mid_lse_elems == 0
+    mfma_ok = a.dtype in (_lib.FTA_F16, _lib.FTA_BF16) and a.head_dim in (64, 128) and pl.rows_per_group >= 16
+    assert pl.kernel == (_lib.KERNEL_MFMA if mfma_ok else _lib.KERNEL_SHUFFLE)
+
+
+def test_plan_headline_shape_fills_the_gpu(fta_lib):
+    """bsz 8 x 8 kv heads x 256 rows: 64 independent streams must be split so that at
+    least one workgroup lands on each of the 256 CUs."""
+    st, pl = plan(fta_lib, base_args())
+    assert st == 0 and pl.kernel == _lib.KERNEL_MFMA
+    assert pl.rows_per_group == 256 and pl.num_workgroups >= 256
+    st, pl4 = plan(fta_lib, base_args(bsz=1, cache_len=131072, v_cache_len=131072))
+    assert pl4.num_workgroups >= 256
+
+
+def test_plan_overrides(fta_lib):
+    st, pl = plan(fta_lib, base_args(force_splits=3))
+    assert st == 0 and pl.num_splits == 3
+    st, pl = plan(fta_lib, base_args(force_kernel=_lib.KERNEL_SHUFFLE))
+    assert st == 0 and pl.kernel == _lib.KERNEL_SHUFFLE and pl.rows_per_wg == 16
+    st, _ = plan(fta_lib, base_args(force_kernel=_lib.KERNEL_MFMA, dtype=_lib.FTA_F32))
+    assert st == -9
+
+
+def test_python_wrapper_rejects_cpu_tensors():
+    """No CPU fallback: the product path refuses CPU tensors outright."""
+    import torch
+    from flash_tree_attn_amd import flash_decoding_attention
+    q = torch.zeros(1, 2, 4, 64)
+    kv = torch.zeros(1, 2, 16, 64)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        flash_decoding_attention(q, kv, kv, q, q, torch.zeros(4, 4), torch.tensor([16]))

@@ -1,0 +1,305 @@
+"""GPU parity: the HIP path (through the C ABI) against the oracle on the same seeded
+inputs. Tolerance for fp16/bf16 is the one the target states: atol 2e-3, rtol 1e-2
+against the fp32 oracle; fp32 inputs are held to atol 2e-5, rtol 1e-4."""
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from flash_tree_attn_amd import _lib, flash_decoding_attention
+from flash_tree_attn_amd.synthetic import CONFIGS, make_inputs
+from flash_tree_attn_amd.tree_mask import additive_mask_from_parents, chain_parents, random_tree_parents
+from oracle.tree_attn_oracle import tree_attention_oracle, two_stage_oracle
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+TOL = {torch.float16: dict(atol=2e-3, rtol=1e-2), torch.bfloat16: dict(atol=2e-3, rtol=1e-2),
+       torch.float32: dict(atol=2e-5, rtol=1e-4)}
+DEV = "cuda"
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _library_is_loaded():
+    _lib.load()  # raises if libfta.so is missing: no silent fallback
+
+
+def make(seed, bsz, hq, hkv, L, D, tmax, dtype, lens=None, cur_heads=None, tree="random"):
+    g = torch.Generator().manual_seed(seed)
+    r = lambda *s: torch.randn(*s, generator=g).to(dtype).to(DEV)
+    ch = hkv if cur_heads is None else cur_heads
+    x = dict(q=r(bsz, hq, L, D), k_cache=r(bsz, hkv, tmax, D), v_cache=r(bsz, hkv, tmax, D),
+             current_k=r(bsz, ch, L, D), current_v=r(bsz, ch, L, D))
+    parents = chain_parents(L) if tree == "chain" else random_tree_parents(L, g)
+    x["mask"] = additive_mask_from_parents(parents, device=DEV)
+    if lens is None:
+        lens = torch.randint(0, tmax + 1, (bsz,), generator=g)
+    x["kv_seq_len"] = torch.as_tensor(lens, dtype=torch.int64).to(DEV)
+    x["kv_group_num"] = hq // hkv
+    return x
+
+
+def oracle(x, sm_scale=None, dtype=torch.float32):
+    return tree_attention_oracle(x["q"], x["k_cache"], x["v_cache"], x["current_k"], x["current_v"], x["mask"],
+                                 x["kv_seq_len"], sm_scale, x["kv_group_num"], dtype=dtype)
+
+
+def run(x, block_size=64, sm_scale=None, **kw):
+    return flash_decoding_attention(x["q"], x["k_cache"], x["v_cache"], x["current_k"], x["current_v"], x["mask"],
+                                    x["kv_seq_len"], block_size, sm_scale=sm_scale, kv_group_num=x["kv_group_num"], **kw)
+
+
+def check(out, ref, dtype):
+    assert out.dtype == dtype
+    assert torch.isfinite(out).all()
+    torch.testing.assert_close(out.float(), ref.float(), **TOL[dtype])
+
+
+# ---------------------------------------------------------------- fixtures
+def test_golden_cfg1_fp32_chain():
+    """BASELINE config 1 (bsz 1, 8 MHA heads, D 64, L 4, chain mask, T 256, fp32)."""
+    x = make_inputs(CONFIGS["cfg1_plumbing_fp32"], seed=0, device=DEV)
+    out = run(x)
+    check(out, oracle(x), torch.float32)
+    data = np.load(os.path.join(GOLDEN, "cfg1_seed0.npz"))
+    import hashlib
+    h = hashlib.sha256()
+    for t in (x["q"], x["k_cache"], x["v_cache"], x["current_k"], x["current_v"]):
+        h.update(t.cpu().contiguous().numpy().tobytes())
+    if h.hexdigest() == str(data["input_digest"]):
+        torch.testing.assert_close(out.cpu().double(), torch.from_numpy(data["out"]), atol=2e-5, rtol=1e-4)
+    for splits in (1, 2, 4):
+        check(run(x, _force_splits=splits), oracle(x), torch.float32)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_golden_tiny_gqa_ragged(dtype):
+    d = np.load(os.path.join(GOLDEN, "tiny_gqa_ragged.npz"))
+    t = lambda n: torch.from_numpy(d[n]).to(DEV)
+    c = lambda n: t(n).to(dtype)
+    out = flash_decoding_attention(c("q"), c("k"), c("v"), c("ck"), c("cv"), t("mask"), t("lens"), 16, kv_group_num=2)
+    if dtype != torch.bfloat16:  # stored values are fp16-representable
+        check(out, t("out"), dtype)
+    else:
+        ref = tree_attention_oracle(c("q"), c("k"), c("v"), c("ck"), c("cv"), t("mask"), t("lens"), None, 2)
+        check(out, ref, dtype)
+
+
+# ---------------------------------------------------------------- BASELINE configs 2-5
+def test_cfg2_medusa_fp16_ragged():
+    cfg = CONFIGS["cfg2_medusa_7b_fp16"]
+    x = make_inputs(cfg, seed=0, device=DEV)
+    check(run(x), oracle(x), cfg.dtype)
+
+
+def test_cfg3_gqa_bf16_full_size():
+    cfg = CONFIGS["cfg3_gqa_8b_bf16"]
+    x = make_inputs(cfg, seed=0, device=DEV, gen_device=DEV)
+    ref = oracle(x)
+    check(run(x), ref, cfg.dtype)
+    for splits in (1, 3, 16):
+        check(run(x, _force_splits=splits), ref, cfg.dtype)
+
+
+def test_cfg4_long_context_bf16_full_size():
+    cfg = CONFIGS["cfg4_long_ctx_bf16"]
+    x = make_inputs(cfg, seed=0, device=DEV, gen_device=DEV)
+    check(run(x), oracle(x), cfg.dtype)
+
+
+def test_cfg5_ragged_70b_bf16_full_size():
+    cfg = CONFIGS["cfg5_ragged_70b_bf16"]
+    x = make_inputs(cfg, seed=0, device=DEV, gen_device=DEV)
+    out = run(x)
+    check(out, oracle(x), cfg.dtype)
+    # the hint only shrinks the grid
+    out_hint = run(x, max_seq_len_in_batch=int(x["kv_seq_len"].max()))
+    check(out_hint, out, cfg.dtype)
+
+
+def test_reference_test_shape_fp16():
+    """The reference's single test (flash_tree_attn.py:416-440): Z 32, H 32, N_CTX 4096,
+    D 128, q_len 128, fp16, block 128, a {1,-inf} mask, tree K/V with num_heads heads,
+    checked there with atol 1e-2."""
+    g = torch.Generator(device=DEV).manual_seed(20)
+    n = lambda *s, std=1.0: (torch.randn(*s, generator=g, device=DEV) * std).half()
+    q, k, v = n(32, 32, 128, 128, std=0.5), n(32, 32, 4096, 128, std=0.5), n(32, 32, 4096, 128, std=0.5)
+    ck, cv = n(32, 32, 128, 128), n(32, 32, 128, 128)
+    allowed = torch.rand(128, 128, generator=g, device=DEV) < 0.5
+    allowed |= torch.eye(128, dtype=torch.bool, device=DEV)
+    mask = torch.where(allowed, torch.ones((), device=DEV), torch.full((), -math.inf, device=DEV))
+    lens = torch.full((32,), 4096, dtype=torch.int64, device=DEV)
+    out = flash_decoding_attention(q, k, v, ck, cv, mask, lens, 128)
+    ref = tree_attention_oracle(q, k, v, ck, cv, mask, lens, None, 1)
+    check(out, ref, torch.float16)
+
+
+# ---------------------------------------------------------------- shape / dtype sweep
+SWEEP = [
+    # bsz hq hkv  L   D   tmax dtype            lens
+    (2, 4, 4, 1, 64, 100, torch.float16, [100, 33]),          # plain decode, one row
+    (2, 8, 2, 3, 128, 300, torch.bfloat16, [300, 1]),         # rows 12 < 16 -> shuffle
+    (1, 8, 2, 4, 128, 200, torch.bfloat16, [200]),            # rows 16 -> MFMA
+    (3, 6, 3, 16, 64, 257, torch.float16, [0, 64, 257]),      # T=0, T multiple, T odd
+    (2, 4, 1, 26, 128, 513, torch.float16, [513, 129]),       # rows 104, padded block
+    (2, 16, 2, 40, 128, 700, torch.bfloat16, [700, 699]),     # rows 320 -> two row blocks
+    (1, 2, 2, 128, 64, 90, torch.bfloat16, [90]),             # L 128: two tree tiles
+    (1, 2, 1, 130, 128, 10, torch.float16, [10]),             # rows 260, ragged tree tiles
+    (2, 4, 2, 8, 32, 150, torch.float16, [150, 20]),          # D 32 -> shuffle
+    (1, 4, 2, 8, 256, 150, torch.bfloat16, [131]),            # D 256 -> shuffle
+    (2, 4, 2, 20, 256, 80, torch.float32, [80, 7]),           # fp32, D 256
+    (1, 2, 2, 33, 32, 64, torch.float32, [64]),               # fp32, D 32, 3 row blocks of 16
+]
+
+
+@pytest.mark.parametrize("case", SWEEP, ids=lambda c: f"b{c[0]}h{c[1]}kv{c[2]}L{c[3]}D{c[4]}T{c[5]}{str(c[6])[6:]}")
+def test_sweep(case):
+    bsz, hq, hkv, L, D, tmax, dtype, lens = case
+    x = make(7, bsz, hq, hkv, L, D, tmax, dtype, lens)
+    ref = oracle(x)
+    check(run(x), ref, dtype)
+    check(run(x, block_size=16, _force_splits=3), ref, dtype)
+    if dtype != torch.float32:
+        # both stage-1 kernels agree with the oracle on the same inputs
+        check(run(x, _force_kernel=_lib.KERNEL_SHUFFLE), ref, dtype)
+
+
+@pytest.mark.parametrize("splits", [1, 2, 5, 13])
+def test_split_count_independence(splits):
+    x = make(11, 3, 8, 2, 24, 128, 1000, torch.bfloat16, [1000, 517, 64])
+    check(run(x, _force_splits=splits), oracle(x), torch.bfloat16)
+
+
+# ---------------------------------------------------------------- argument contract
+def test_mask_forms():
+    x = make(13, 2, 4, 2, 18, 128, 120, torch.float16, [120, 50])
+    ref = oracle(x)
+    base = x["mask"]
+    for m in (base, base[None, None], base[None, None].expand(2, 4, 18, 18).contiguous(),
+              base[None, None].expand(2, 1, 18, 18).contiguous(), torch.isfinite(base), base.half()):
+        x["mask"] = m
+        check(run(x), ref, torch.float16)
+    # per-batch, per-head masks really are indexed per batch and head
+    g = torch.Generator().manual_seed(5)
+    per = torch.stack([torch.stack([additive_mask_from_parents(random_tree_parents(18, g)) for _ in range(4)])
+                       for _ in range(2)]).to(DEV)
+    x["mask"] = per
+    check(run(x), oracle(x), torch.float16)
+    # additive semantics: {1,-inf} like the reference's generator (flash_tree_attn.py:403-414)
+    x["mask"] = torch.where(torch.isfinite(base), torch.ones_like(base), base)
+    check(run(x), oracle(x), torch.float16)
+    # arbitrary finite bias
+    x["mask"] = torch.randn(18, 18, generator=g).to(DEV)
+    check(run(x), oracle(x), torch.float16)
+
+
+def test_fully_masked_rows_and_empty_cache():
+    x = make(17, 2, 4, 2, 20, 128, 64, torch.bfloat16, [0, 40])
+    x["mask"] = x["mask"].clone()
+    x["mask"][3, :] = -math.inf
+    ref = oracle(x)
+    assert torch.all(ref[0, :, 3] == 0)
+    for kern in (-1, _lib.KERNEL_SHUFFLE):
+        out = run(x, _force_kernel=kern)
+        check(out, ref, torch.bfloat16)
+        assert torch.all(out[0, :, 3] == 0)
+
+
+def test_tree_heads_per_query_head():
+    """current_k/current_v with num_heads heads (flash_tree_attn.py:424-425) under GQA."""
+    x = make(19, 2, 8, 2, 16, 128, 200, torch.float16, [200, 77], cur_heads=8)
+    check(run(x), oracle(x), torch.float16)
+
+
+def test_strided_views_like_reference_benchmark():
+    """flash_tree_attn.py:471-483 passes k[:, :, :N] and k[:, :, N:] of one buffer."""
+    g = torch.Generator().manual_seed(23)
+    Z, H, N, L, D = 2, 4, 192, 16, 128
+    q = torch.randn(Z, H, L, D, generator=g).half().to(DEV)
+    k = torch.randn(Z, H, N + L, D, generator=g).half().to(DEV)
+    v = torch.randn(Z, H, N + L, D, generator=g).half().to(DEV)
+    mask = additive_mask_from_parents(random_tree_parents(L, g), device=DEV)
+    lens = torch.tensor([N] * Z, device=DEV)
+    out = flash_decoding_attention(q, k[:, :, :N], v[:, :, :N], k[:, :, N:], v[:, :, N:], mask, lens,
+                                   block_size=64, sm_scale=0.11)
+    ref = tree_attention_oracle(q, k[:, :, :N], v[:, :, :N], k[:, :, N:], v[:, :, N:], mask, lens, 0.11, 1)
+    check(out, ref, torch.float16)
+    # a transposed (inner stride != 1) q is copied, not rejected
+    qt = q.transpose(2, 3).contiguous().transpose(2, 3)
+    check(flash_decoding_attention(qt, k[:, :, :N], v[:, :, :N], k[:, :, N:], v[:, :, N:], mask, lens, sm_scale=0.11),
+          ref, torch.float16)
+
+
+def test_user_buffers_reference_sized():
+    """output / mid_output / mid_output_lse shaped as the reference allocates them
+    (flash_tree_attn.py:276-284) are accepted; output receives the final result."""
+    x = make(29, 2, 8, 2, 32, 128, 2048, torch.bfloat16, [2048, 1000])
+    kv_max_split = -(-2048 // 64)
+    out = torch.empty(2, 8, 32, 128, dtype=torch.bfloat16, device=DEV)
+    mid = torch.empty(2, 8, kv_max_split, 32, 128, dtype=torch.float32, device=DEV)
+    lse = torch.empty(2, 8, kv_max_split, 32, dtype=torch.float32, device=DEV)
+    ret = run(x, output=out, mid_output=mid, mid_output_lse=lse, max_seq_len_in_batch=2048)
+    assert ret.data_ptr() == out.data_ptr()
+    check(out, oracle(x), torch.bfloat16)
+    # scratch too small for the planned splits -> the reference's assert (flash_tree_attn.py:286-288)
+    with pytest.raises(AssertionError):
+        run(x, mid_output=mid[:, :, :1], mid_output_lse=lse[:, :, :1], _force_splits=4)
+
+
+def test_errors_like_reference_asserts():
+    x = make(31, 1, 2, 2, 4, 64, 32, torch.float16, [32])
+    with pytest.raises(AssertionError):
+        run(x, block_size=48)                       # flash_tree_attn.py:268
+    bad = dict(x)
+    bad["v_cache"] = x["v_cache"][:, :, :16]
+    with pytest.raises(AssertionError):
+        run(bad)                                    # flash_tree_attn.py:264
+    bad = make(31, 1, 2, 2, 4, 64, 32, torch.float16, [32])
+    for name in ("q", "k_cache", "v_cache", "current_k", "current_v"):
+        bad[name] = torch.cat([bad[name], bad[name][..., :32]], dim=-1)
+    with pytest.raises(AssertionError):
+        run(bad)                                    # head_dim 96: flash_tree_attn.py:263
+
+
+def test_int32_lengths_scale_override_and_negative_scale():
+    x = make(37, 2, 4, 2, 16, 64, 99, torch.float16, [99, 12])
+    ref = oracle(x, sm_scale=0.05)
+    check(run(x, sm_scale=0.05), ref, torch.float16)
+    x32 = dict(x)
+    x32["kv_seq_len"] = x["kv_seq_len"].int()
+    check(run(x32, sm_scale=0.05), ref, torch.float16)
+    check(run(x, sm_scale=-0.07), oracle(x, sm_scale=-0.07), torch.float16)
+
+
+def test_lengths_beyond_cache_are_clamped_and_padding_is_ignored():
+    x = make(41, 2, 4, 2, 16, 128, 128, torch.bfloat16, [100, 128])
+    ref = oracle(x)
+    # poison the padding past kv_seq_len: it must never be read into the result
+    x["k_cache"][0, :, 100:] = float("nan")
+    x["v_cache"][0, :, 100:] = float("inf")
+    check(run(x), ref, torch.bfloat16)
+
+
+# ---------------------------------------------------------------- size-independent properties
+def test_properties_at_headline_size():
+    cfg = CONFIGS["cfg3_gqa_8b_bf16"]
+    x = make_inputs(cfg, seed=1, device=DEV, gen_device=DEV)
+    # constant V -> constant output, whatever the logits are
+    xc = dict(x)
+    xc["v_cache"] = torch.full_like(x["v_cache"], 0.75)
+    xc["current_v"] = torch.full_like(x["current_v"], 0.75)
+    out = run(xc)
+    torch.testing.assert_close(out.float(), torch.full_like(out, 0.75).float(), atol=4e-3, rtol=0)
+    # q = 0 -> mean over cache and allowed tree values
+    xz = dict(x)
+    xz["q"] = torch.zeros_like(x["q"])
+    out = run(xz).float()
+    allowed = torch.isfinite(x["mask"]).float()                          # [L, L]
+    num = x["v_cache"].float().sum(2)[:, :, None] + torch.einsum("ij,bhjd->bhid", allowed, x["current_v"].float())
+    mean = (num / (cfg.cache_len + allowed.sum(1))[None, None, :, None]).repeat_interleave(cfg.kv_group_num, dim=1)
+    torch.testing.assert_close(out, mean, atol=2e-3, rtol=1e-2)
+    # output is linear in V for fixed q, k
+    x2 = dict(x)
+    x2["v_cache"], x2["current_v"] = x["v_cache"] * 2, x["current_v"] * 2
+    torch.testing.assert_close(run(x2).float(), run(x).float() * 2, atol=2e-3, rtol=1e-2)
