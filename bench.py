@@ -1,0 +1,167 @@
+#!/usr/bin/env python3
+"""Benchmark of the tree-attention decode hot path on one MI355X.
+
+A step is one call of `flash_decoding_attention` (stage 1 + LSE merge) on one batch of
+synthetic input already resident in HBM. Steps rotate over several independent KV-cache
+sets so the footprint exceeds the 256 MB Infinity Cache. Prints ONE JSON line:
+value = achieved GB/s over the whole call (algorithmic bytes / time per call),
+`roofline` = the dominant kernel (stage 1) timed alone with HIP events on the launch
+stream, `cpu_baseline` = the fp32 PyTorch eager oracle on the host cores (a bounded
+sample), timed in the same run.
+"""
+import argparse
+import json
+import os
+import re
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", default="cfg3_gqa_8b_bf16", help="workload name (flash_tree_attn_amd.synthetic.CONFIGS)")
+    ap.add_argument("--kv-sets", type=int, default=0, help="independent KV caches to rotate over (0 = enough for >1 GiB)")
+    ap.add_argument("--splits", type=int, default=0, help="pin the split count (0 = heuristic)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
+    return ap.parse_args()
+
+
+def traffic_from_profiles(config_name):
+    """HBM bytes per stage-1 launch from the committed rocprofv3 --pmc summary, if any."""
+    path = os.path.join(ROOT, "profiles", f"stage1_{config_name}_pmc.txt")
+    if not os.path.exists(path):
+        return None
+    m = re.search(r"^traffic_bytes_per_launch:\s*([0-9.eE+]+)", open(path).read(), flags=re.M)
+    return float(m.group(1)) if m else None
+
+
+def cpu_baseline(cfg, x, budget_s):
+    """fp32 eager oracle on the host cores over as many whole sequences of the batch as
+    fit the time budget; reported in the metric's unit (algorithmic GB/s)."""
+    import torch
+    from flash_tree_attn_amd.synthetic import algorithmic_bytes
+    from oracle.tree_attn_oracle import tree_attention_oracle
+
+    cpu = {k: (v.cpu() if torch.is_tensor(v) else v) for k, v in x.items() if k not in ("k_caches", "v_caches")}
+
+    def run(nseq):
+        sl = slice(0, nseq)
+        t0 = time.perf_counter()
+        tree_attention_oracle(cpu["q"][sl], cpu["k_cache"][sl], cpu["v_cache"][sl], cpu["current_k"][sl],
+                              cpu["current_v"][sl], cpu["mask"], cpu["kv_seq_len"][sl], cpu["sm_scale"],
+                              cpu["kv_group_num"])
+        return time.perf_counter() - t0
+
+    run(1)  # warm-up (thread pool, allocator)
+    t1 = run(1)
+    nseq = int(max(1, min(cfg.bsz, budget_s / 2 / max(t1, 1e-6))))
+    reps, times = 0, []
+    t_start = time.perf_counter()
+    while reps < 5 and (reps < 1 or time.perf_counter() - t_start < budget_s):
+        times.append(run(nseq))
+        reps += 1
+    t = sorted(times)[len(times) // 2]
+    sample_cfg_bytes = algorithmic_bytes(cfg, cpu["kv_seq_len"][:nseq], cpu["mask"]) * 1.0
+    # per-sequence terms scale with nseq; recompute q/out/current terms for the sample
+    esz = cpu["q"].element_size()
+    per_seq_fixed = (2 * cfg.num_kv_heads + 2 * cfg.num_heads) * cfg.q_len * cfg.head_dim * esz + 8
+    sample_bytes = sample_cfg_bytes - (cfg.bsz - nseq) * per_seq_fixed
+    return {
+        "value": sample_bytes / t / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"{nseq} of {cfg.bsz} sequences of {cfg.name}, fp32 eager oracle, median of {reps} run(s), "
+                  f"{t * 1e6 / nseq * cfg.bsz:.0f} us/call extrapolated to the full batch, os.cpu_count()={os.cpu_count()}",
+        "us_per_call_extrapolated": t * 1e6 / nseq * cfg.bsz,
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU only: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from flash_tree_attn_amd import _lib, prepare
+    from flash_tree_attn_amd.synthetic import CONFIGS, algorithmic_bytes, flops, make_inputs
+
+    _lib.load()  # no fallback: fail loudly if the HIP library is missing
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    cfg = CONFIGS[args.config]
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    esz = torch.empty((), dtype=cfg.dtype).element_size()
+    kv_bytes = 2 * cfg.bsz * cfg.num_kv_heads * cfg.cache_len * cfg.head_dim * esz
+    kv_sets = args.kv_sets or max(2, min(8, -(-(1 << 30) // kv_bytes)))
+    small = kv_bytes * kv_sets < (64 << 20)
+    x = make_inputs(cfg, seed=0, device=dev, gen_device="cpu" if small else dev, kv_sets=kv_sets)
+
+    calls = [prepare(x["q"], kc, vc, x["current_k"], x["current_v"], x["mask"], x["kv_seq_len"], cfg.block_size,
+                     None, None, None, None, x["sm_scale"], cfg.kv_group_num, _force_splits=args.splits)
+             for kc, vc in zip(x["k_caches"], x["v_caches"])]
+    plan = calls[0].plan
+    nbytes = algorithmic_bytes(cfg, x["kv_seq_len"].cpu(), x["mask"])
+    nflops = flops(cfg, x["kv_seq_len"].cpu())
+
+    # quick self-check of the measured path against the oracle on one sequence
+    from oracle.tree_attn_oracle import tree_attention_oracle
+    out = calls[0].run()
+    ref = tree_attention_oracle(x["q"][:1], x["k_cache"][:1], x["v_cache"][:1], x["current_k"][:1], x["current_v"][:1],
+                                x["mask"], x["kv_seq_len"][:1], x["sm_scale"], cfg.kv_group_num)
+    tol = dict(atol=2e-3, rtol=1e-2) if cfg.dtype != torch.float32 else dict(atol=2e-5, rtol=1e-4)
+    torch.testing.assert_close(out[:1].float(), ref, **tol)
+
+    stream = torch.cuda.current_stream()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def timed(fn_name, steps):
+        torch.cuda.synchronize()
+        e0.record(stream)
+        for i in range(steps):
+            getattr(calls[i % kv_sets], fn_name)()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps  # ms per step
+
+    for i in range(args.warmup):
+        calls[i % kv_sets].run()
+    ms = timed("run", args.steps)
+    ms_stage1 = timed("run_stage1", args.steps)
+    ms_stage2 = timed("run_stage2", args.steps) if plan.num_splits > 1 else 0.0
+
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    gbs_s1 = nbytes / (ms_stage1 * 1e-3) / 1e9
+    result = {
+        "metric": "tree-attn us/call + achieved HBM GB/s (% peak), 8B GQA q_len=64 @8K ctx",
+        "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "us_per_call": ms * 1e3, "pct_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}[cfg.dtype],
+        "data": "synthetic (seed 0, N(0,1) q/k/v, random tree mask), inputs resident in HBM",
+        "config": {"workload": cfg.name, "bsz": cfg.bsz, "q_heads": cfg.num_heads, "kv_heads": cfg.num_kv_heads,
+                   "head_dim": cfg.head_dim, "q_len": cfg.q_len, "cache_len": cfg.cache_len, "lengths": cfg.lengths,
+                   "block_size": cfg.block_size, "kv_sets_rotated": kv_sets, "num_splits": plan.num_splits,
+                   "chunk": plan.chunk, "stage1_kernel": "mfma" if plan.kernel == _lib.KERNEL_MFMA else "shuffle",
+                   "stage1_workgroups": plan.num_workgroups, "algorithmic_bytes": nbytes, "flops": nflops},
+        "tflops": nflops / (ms * 1e-3) / 1e12,
+        "roofline": {"bound": "hbm", "kernel": "stage1", "achieved": round(gbs_s1, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(gbs_s1 / HBM_PEAK_GBS, 4), "traffic": traffic_from_profiles(cfg.name),
+                     "us_per_launch": ms_stage1 * 1e3, "stage2_us_per_launch": ms_stage2 * 1e3,
+                     "mfma_tflops": nflops / (ms_stage1 * 1e-3) / 1e12},
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(cfg, x, args.cpu_seconds)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

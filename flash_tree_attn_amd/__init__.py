@@ -4,10 +4,10 @@ The public function mirrors NonvolatileMemory/flash_tree_attn's
 `flash_decoding_attention` (flash_tree_attn.py:216-231) and calls hand-written HIP
 kernels through the C ABI declared in include/fta.h.
 """
-from .flash_decoding import FtaAssertionError, flash_decoding_attention
+from .flash_decoding import FtaAssertionError, PreparedCall, flash_decoding_attention, prepare
 from .tree_mask import additive_mask_from_parents, ancestor_matrix, chain_parents, random_tree_parents
 
 __all__ = [
-    "flash_decoding_attention", "FtaAssertionError",
+    "flash_decoding_attention", "prepare", "PreparedCall", "FtaAssertionError",
     "additive_mask_from_parents", "ancestor_matrix", "chain_parents", "random_tree_parents",
 ]

@@ -13,7 +13,8 @@ FTA_I32, FTA_I64 = 0, 1
 KERNEL_SHUFFLE, KERNEL_MFMA = 0, 1
 
 EXPORTED_SYMBOLS = (
-    "fta_abi_version", "fta_strerror", "fta_validate", "fta_plan", "fta_decode", "fta_device_cus",
+    "fta_abi_version", "fta_strerror", "fta_validate", "fta_plan", "fta_decode", "fta_decode_stage1",
+    "fta_decode_stage2", "fta_device_cus",
 )
 
 # status -> Python exception class
@@ -73,6 +74,10 @@ def load() -> C.CDLL:
     lib.fta_plan.argtypes = [C.POINTER(FtaArgs), C.c_int, C.POINTER(FtaPlanOut)]
     lib.fta_decode.restype = C.c_int
     lib.fta_decode.argtypes = [C.POINTER(FtaArgs), C.c_void_p]
+    for name in ("fta_decode_stage1", "fta_decode_stage2"):
+        fn = getattr(lib, name)
+        fn.restype = C.c_int
+        fn.argtypes = [C.POINTER(FtaArgs), C.c_void_p]
     lib.fta_device_cus.restype = C.c_int
     if lib.fta_abi_version() != ABI_VERSION:
         raise ImportError(f"libfta.so has ABI {lib.fta_abi_version()}, binding expects {ABI_VERSION}; rebuild it")

@@ -175,7 +175,9 @@ int fta_device_cus(void) {
   return cus;
 }
 
-int fta_decode(const fta_args* args, void* hip_stream) {
+namespace {
+// stages: bit 0 = stage 1, bit 1 = stage 2
+int decode_impl(const fta_args* args, void* hip_stream, int stages) {
   if (!args) return FTA_ERR_NULL_POINTER;
   const fta_args& a = *args;
   if (int st = fta::validate(a)) return st;
@@ -215,11 +217,18 @@ int fta_decode(const fta_args* args, void* hip_stream) {
   }
   for (int i = 0; i < 4; ++i) p.mid_o_stride[i] = a.mid_o_stride[i];
 
-  int st = pl.kernel == FTA_KERNEL_MFMA ? fta::launch_stage1_mfma(p, a.dtype, a.head_dim, hip_stream)
-                                        : fta::launch_stage1_shuffle(p, a.dtype, a.head_dim, hip_stream);
+  int st = FTA_OK;
+  if (stages & 1)
+    st = pl.kernel == FTA_KERNEL_MFMA ? fta::launch_stage1_mfma(p, a.dtype, a.head_dim, hip_stream)
+                                      : fta::launch_stage1_shuffle(p, a.dtype, a.head_dim, hip_stream);
   if (st) return st;
-  if (pl.num_splits > 1) st = fta::launch_stage2_merge(p, a.dtype, a.head_dim, hip_stream);
+  if ((stages & 2) && pl.num_splits > 1) st = fta::launch_stage2_merge(p, a.dtype, a.head_dim, hip_stream);
   return st;
 }
+}  // namespace
+
+int fta_decode(const fta_args* args, void* hip_stream) { return decode_impl(args, hip_stream, 3); }
+int fta_decode_stage1(const fta_args* args, void* hip_stream) { return decode_impl(args, hip_stream, 1); }
+int fta_decode_stage2(const fta_args* args, void* hip_stream) { return decode_impl(args, hip_stream, 2); }
 
 }  // extern "C"

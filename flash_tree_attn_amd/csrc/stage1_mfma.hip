@@ -51,15 +51,16 @@ struct MfmaSmem {
   static constexpr int kTotal = 2 * (kKBuf + kVBuf);
 };
 
-// max over the two half-waves: lanes i and i+32 hold the same query row.
-__device__ __forceinline__ float half_swap_max(float x) {
+// Lanes i and i+32 hold the same query row. v_permlane32_swap exchanges the upper half
+// of its first operand with the lower half of its second; the partner's value is then
+// in result 1 for lanes < 32 and in result 0 for lanes >= 32 (also when the compiler
+// assigns both operands the same register, where both results hold the partner).
+__device__ __forceinline__ float half_partner(float x, int lh) {
   auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, x), __builtin_bit_cast(unsigned, x), false, false);
-  return fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
+  return __builtin_bit_cast(float, lh ? r[0] : r[1]);
 }
-__device__ __forceinline__ float half_swap_sum(float x) {
-  auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, x), __builtin_bit_cast(unsigned, x), false, false);
-  return __builtin_bit_cast(float, r[0]) + __builtin_bit_cast(float, r[1]);
-}
+__device__ __forceinline__ float half_swap_max(float x, int lh) { return fmaxf(x, half_partner(x, lh)); }
+__device__ __forceinline__ float half_swap_sum(float x, int lh) { return x + half_partner(x, lh); }
 
 template <typename T, int D, int QB, int NW>
 __global__ void __launch_bounds__(NW * 64) stage1_mfma_kernel(const KernelParams p) {
@@ -238,7 +239,7 @@ __global__ void __launch_bounds__(NW * 64) stage1_mfma_kernel(const KernelParams
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[kb][qb][r]);
-      mx = half_swap_max(mx);
+      mx = half_swap_max(mx, lh);
       m_new = fmaxf(m_old, masked ? mx : mx * c);
       m_use = (m_new == neg_inf()) ? 0.f : m_new;
       const float alpha = fast_exp2(m_old - m_use);
@@ -263,24 +264,47 @@ __global__ void __launch_bounds__(NW * 64) stage1_mfma_kernel(const KernelParams
       for (int kk = 0; kk < 4; ++kk) {
         Vec8 pk;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) pk[e] = static_cast<T>(s[kk >> 1][qb][(kk & 1) * 8 + e]);
+        for (int e = 0; e < 8; ++e) {
+          const float pv = s[kk >> 1][qb][(kk & 1) * 8 + e];
+          pk[e] = static_cast<T>(pv);
+          // masked tiles keep the rounding residue for a second, compensating product
+          if (masked) s[kk >> 1][qb][(kk & 1) * 8 + e] = pv - static_cast<float>(pk[e]);
+        }
         pf[qb][kk] = pk;
       }
     }
 
     // ---- O^T += V^T P^T
+    auto pv_product = [&]() {
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
+      for (int kk = 0; kk < 4; ++kk) {
 #pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        const char* va = Vb + v_rd + (kk * 16) * SM::kVPitch + db * 64;
-        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 FTA_LDS*)(va));
-        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 FTA_LDS*)(va + 8 * SM::kVPitch));
-        const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        const Vec8 a = __builtin_bit_cast(Vec8, both);
+        for (int db = 0; db < DB; ++db) {
+          const char* va = Vb + v_rd + (kk * 16) * SM::kVPitch + db * 64;
+          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 FTA_LDS*)(va));
+          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 FTA_LDS*)(va + 8 * SM::kVPitch));
+          const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          const Vec8 a = __builtin_bit_cast(Vec8, both);
 #pragma unroll
-        for (int qb = 0; qb < QB; ++qb) o[db][qb] = M::mma(a, pf[qb][kk], o[db][qb]);
+          for (int qb = 0; qb < QB; ++qb) o[db][qb] = M::mma(a, pf[qb][kk], o[db][qb]);
+        }
       }
+    };
+    pv_product();
+    if (masked) {
+      // Tree tiles and the ragged last cache tile are where single keys can carry large
+      // weights (short sequences); a second product with the low-order part of P removes
+      // the 2^-9 rounding of P there. Full cache tiles use one product.
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+          Vec8 pk;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) pk[e] = static_cast<T>(s[kk >> 1][qb][(kk & 1) * 8 + e]);
+          pf[qb][kk] = pk;
+        }
+      pv_product();
     }
   }
 
@@ -290,7 +314,7 @@ __global__ void __launch_bounds__(NW * 64) stage1_mfma_kernel(const KernelParams
   const bool direct = p.num_splits == 1;
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
-    const float l_tot = half_swap_sum(l_run[qb]);
+    const float l_tot = half_swap_sum(l_run[qb], lh);
     if (!row_ok[qb]) continue;
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
     const int head = row_head[qb], i = row_i[qb];

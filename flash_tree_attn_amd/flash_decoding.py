@@ -145,34 +145,41 @@ def plan_for(args: "_lib.FtaArgs", num_cus: int) -> "_lib.FtaPlanOut":
     return pl
 
 
-def flash_decoding_attention(
-    q: torch.Tensor,
-    k_cache: torch.Tensor,
-    v_cache: torch.Tensor,
-    current_k: torch.Tensor,
-    current_v: torch.Tensor,
-    mask: torch.Tensor,
-    kv_seq_len: torch.Tensor,
-    block_size: int = 64,
-    max_seq_len_in_batch: Optional[int] = None,
-    output: Optional[torch.Tensor] = None,
-    mid_output: Optional[torch.Tensor] = None,
-    mid_output_lse: Optional[torch.Tensor] = None,
-    sm_scale: Optional[float] = None,
-    kv_group_num: int = 1,
-    *,
-    _force_splits: int = 0,
-    _force_kernel: int = -1,
-) -> torch.Tensor:
-    """Tree-attention decode (speculative-decoding verification).
+class PreparedCall:
+    """One validated, planned call: the filled fta_args, its output and scratch tensors.
+    `run()` launches the whole path on the current stream; `run_stage1()` / `run_stage2()`
+    launch the halves (a profiler or a KV-sequence-sharded caller uses those). The tensors
+    it was prepared from must stay alive and unmoved while it is in use."""
 
-    Same parameters, order and defaults as the reference (flash_tree_attn.py:216-231):
-      q [bsz, num_heads, q_len, head_dim]; k_cache / v_cache [bsz, num_kv_heads, ctx, head_dim];
-      current_k / current_v [bsz, num_kv_heads, q_len, head_dim]; mask [q_len, q_len] or
-      [bsz, num_heads, q_len, q_len], ADDED to the tree logits; kv_seq_len [bsz].
-    Returns [bsz, num_heads, q_len, head_dim] in q's dtype.
-    """
-    lib = _lib.load()
+    def __init__(self, args, plan, output, mid_output, mid_output_lse, keep, device):
+        self.args, self.plan, self.output = args, plan, output
+        self.mid_output, self.mid_output_lse = mid_output, mid_output_lse
+        self._keep, self._device = keep, device
+        self._lib = _lib.load()
+        self._ref = C.byref(args)
+
+    def _launch(self, fn):
+        with torch.cuda.device(self._device):
+            stream = torch.cuda.current_stream(self._device).cuda_stream
+            _check(fn(self._ref, C.c_void_p(stream)))
+        return self.output
+
+    def run(self):
+        return self._launch(self._lib.fta_decode)
+
+    def run_stage1(self):
+        return self._launch(self._lib.fta_decode_stage1)
+
+    def run_stage2(self):
+        return self._launch(self._lib.fta_decode_stage2)
+
+
+def prepare(q, k_cache, v_cache, current_k, current_v, mask, kv_seq_len, block_size=64,
+            max_seq_len_in_batch=None, output=None, mid_output=None, mid_output_lse=None,
+            sm_scale=None, kv_group_num=1, _force_splits=0, _force_kernel=-1) -> PreparedCall:
+    """Validates, plans and allocates once; the returned PreparedCall can be launched
+    repeatedly (a decode loop that reuses its buffers pays the Python checks once)."""
+    _lib.load()
     args, keep = build_args(q, k_cache, v_cache, current_k, current_v, mask, kv_seq_len, block_size,
                             max_seq_len_in_batch, sm_scale, kv_group_num, _force_splits, _force_kernel)
     bsz, hq, L, D = q.shape
@@ -205,9 +212,38 @@ def flash_decoding_attention(
         args.mid_splits = min(mid_output.size(2), mid_output_lse.size(2))
         args.mid_o_stride[:] = mid_output.stride()[:4]
         args.mid_lse_stride[:] = mid_output_lse.stride()[:3]
+        if args.mid_splits < pl.num_splits:
+            _check(-5)
+    return PreparedCall(args, pl, output, mid_output, mid_output_lse, keep, dev)
 
-    with torch.cuda.device(dev):
-        stream = torch.cuda.current_stream(dev).cuda_stream
-        _check(lib.fta_decode(C.byref(args), C.c_void_p(stream)))
-    del keep
-    return output
+
+def flash_decoding_attention(
+    q: torch.Tensor,
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    current_k: torch.Tensor,
+    current_v: torch.Tensor,
+    mask: torch.Tensor,
+    kv_seq_len: torch.Tensor,
+    block_size: int = 64,
+    max_seq_len_in_batch: Optional[int] = None,
+    output: Optional[torch.Tensor] = None,
+    mid_output: Optional[torch.Tensor] = None,
+    mid_output_lse: Optional[torch.Tensor] = None,
+    sm_scale: Optional[float] = None,
+    kv_group_num: int = 1,
+    *,
+    _force_splits: int = 0,
+    _force_kernel: int = -1,
+) -> torch.Tensor:
+    """Tree-attention decode (speculative-decoding verification).
+
+    Same parameters, order and defaults as the reference (flash_tree_attn.py:216-231):
+      q [bsz, num_heads, q_len, head_dim]; k_cache / v_cache [bsz, num_kv_heads, ctx, head_dim];
+      current_k / current_v [bsz, num_kv_heads, q_len, head_dim]; mask [q_len, q_len] or
+      [bsz, num_heads, q_len, q_len], ADDED to the tree logits; kv_seq_len [bsz].
+    Returns [bsz, num_heads, q_len, head_dim] in q's dtype.
+    """
+    return prepare(q, k_cache, v_cache, current_k, current_v, mask, kv_seq_len, block_size,
+                   max_seq_len_in_batch, output, mid_output, mid_output_lse, sm_scale, kv_group_num,
+                   _force_splits, _force_kernel).run()

@@ -137,6 +137,15 @@ int fta_plan(const fta_args* args, int num_cus, fta_plan_out* plan);
  * the default stream). Replaces flash_tree_attn.py:293-376. Asynchronous. */
 int fta_decode(const fta_args* args, void* hip_stream);
 
+/* The two halves of fta_decode, for callers that place something between them: a
+ * deployment that shards the KV sequence over devices runs stage 1 on each shard,
+ * exchanges the fp32 partials (mid_o, mid_lse) and runs stage 2 on the gathered set;
+ * a profiler times them separately. fta_decode_stage1 replaces flash_tree_attn.py:
+ * 295-334 and :367-373 (with one split it writes `out` directly and stage 2 is a
+ * no-op); fta_decode_stage2 replaces flash_tree_attn.py:339-365. */
+int fta_decode_stage1(const fta_args* args, void* hip_stream);
+int fta_decode_stage2(const fta_args* args, void* hip_stream);
+
 /* Number of compute units of the current HIP device, or a negative fta_status. */
 int fta_device_cus(void);
 
