@@ -20,6 +20,9 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    # NaN-agnostic min/max (no canonicalising v_max x,x,x); infinities stay honoured,
+    # the kernels use -inf as the "masked" logit.
+    "-fno-honor-nans",
     "-I", INCLUDE, "-I", CSRC,
 ]
 

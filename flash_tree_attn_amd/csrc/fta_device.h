@@ -7,6 +7,7 @@
 
 namespace fta {
 
+typedef __attribute__((ext_vector_type(2))) float f32x2;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
@@ -42,13 +43,32 @@ struct WorkItem {
   int split, unit, batch, row_block;
 };
 
-// Linear workgroup id -> (split, row_block, unit, batch), split fastest.
+// Linear workgroup id -> (split, row_block, unit, batch).
+// Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2. The row
+// blocks of one (batch, unit, split) read the same K/V stream, so they are given ids
+// that differ by a multiple of 8 and land on the same XCD: the second block's K/V
+// fetches hit in L2 instead of going to HBM again. Groups beyond the last multiple of
+// 8 fall back to consecutive ids.
 __device__ __forceinline__ WorkItem decode_work(const KernelParams& p, int id) {
+  constexpr int kXcds = 8;
+  const int rb_n = p.row_blocks;
+  const int groups = p.num_splits * p.units * p.bsz;
+  const int even_groups = groups - groups % kXcds;
+  int g, rb;
+  if (id < even_groups * rb_n) {
+    const int xcd = id % kXcds, j = id / kXcds;
+    rb = j % rb_n;
+    g = (j / rb_n) * kXcds + xcd;
+  } else {
+    const int r = id - even_groups * rb_n;
+    rb = r % rb_n;
+    g = even_groups + r / rb_n;
+  }
   WorkItem w;
-  w.split = id % p.num_splits; id /= p.num_splits;
-  w.row_block = id % p.row_blocks; id /= p.row_blocks;
-  w.unit = id % p.units;
-  w.batch = id / p.units;
+  w.row_block = rb;
+  w.split = g % p.num_splits; g /= p.num_splits;
+  w.unit = g % p.units;
+  w.batch = g / p.units;
   return w;
 }
 

@@ -10,7 +10,14 @@
 
 namespace fta {
 
-int mfma_rows_per_wg(int rows) { return rows > 128 ? 256 : 128; }
+// One MFMA workgroup holds 128 query rows (4 waves x 32). Two such workgroups share a
+// CU; they synchronise independently, so one's softmax overlaps the other's MFMAs.
+// FTA_ROWS_PER_WG=256 selects the 8-wave, 256-row variant (tuning only).
+int mfma_rows_per_wg(int rows) {
+  if (const char* env = std::getenv("FTA_ROWS_PER_WG"))
+    if (std::atoi(env) == 256 && rows > 128) return 256;
+  return 128;
+}
 
 namespace {
 

@@ -18,6 +18,8 @@
 // (current_k / current_v with the additive mask), which replaces the eager block and
 // sigmoid merge of flash_tree_attn.py:367-373. Output: the final result (one split)
 // or a normalised fp32 partial plus its log-sum-exp (flash_tree_attn.py:121-144).
+#include <type_traits>
+
 #include "fta_device.h"
 
 namespace fta {
@@ -27,6 +29,7 @@ template <typename T> struct Mfma;
 template <> struct Mfma<__bf16> {
   using Vec8 = bf16x8;
   using Vec4 = bf16x4;
+  using Vec2 = bf16x2;
   static __device__ __forceinline__ f32x16 mma(Vec8 a, Vec8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
@@ -34,6 +37,7 @@ template <> struct Mfma<__bf16> {
 template <> struct Mfma<_Float16> {
   using Vec8 = f16x8;
   using Vec4 = f16x4;
+  using Vec2 = f16x2;
   static __device__ __forceinline__ f32x16 mma(Vec8 a, Vec8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
@@ -45,7 +49,7 @@ typedef __attribute__((ext_vector_type(8))) short s16x8;
 template <int D>
 struct MfmaSmem {
   static constexpr int kKPitch = D * 2 + 16;  // bytes; +16 keeps row-per-lane 128-bit reads conflict free
-  static constexpr int kVPitch = D * 2 + 16;
+  static constexpr int kVPitch = D * 2 + 64;  // bytes; +64 spreads the 4 key rows of a transposing read over all banks
   static constexpr int kKBuf = kKeyTile * kKPitch;
   static constexpr int kVBuf = kKeyTile * kVPitch;
   static constexpr int kTotal = 2 * (kKBuf + kVBuf);
@@ -63,7 +67,8 @@ __device__ __forceinline__ float half_swap_max(float x, int lh) { return fmaxf(x
 __device__ __forceinline__ float half_swap_sum(float x, int lh) { return x + half_partner(x, lh); }
 
 template <typename T, int D, int QB, int NW>
-__global__ void __launch_bounds__(NW * 64) stage1_mfma_kernel(const KernelParams p) {
+__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(QB == 1 ? 2 : 1, QB == 1 ? 2 : 1)))
+stage1_mfma_kernel(const KernelParams p) {
   using M = Mfma<T>;
   using Vec8 = typename M::Vec8;
   using SM = MfmaSmem<D>;
@@ -146,7 +151,7 @@ __global__ void __launch_bounds__(NW * 64) stage1_mfma_kernel(const KernelParams
   const int ld_row = tid / kChunks;
   const int ld_chunk = tid % kChunks;
   u32x4 kreg[kPasses], vreg[kPasses];
-  auto issue_loads = [&](int t) {
+  auto issue_loads = [&](int t) __attribute__((always_inline)) {
     const bool tree = t >= cache_tiles;
     const int key0 = tree ? (t - cache_tiles) * kKeyTile : kv_start + t * kKeyTile;
     const int key_lim = tree ? L : kv_end;
@@ -166,7 +171,7 @@ __global__ void __launch_bounds__(NW * 64) stage1_mfma_kernel(const KernelParams
       vreg[ps] = vq;
     }
   };
-  auto store_lds = [&](int buf) {
+  auto store_lds = [&](int buf) __attribute__((always_inline)) {
     char* kdst = smem + buf * SM::kKBuf;
     char* vdst = smem + 2 * SM::kKBuf + buf * SM::kVBuf;
 #pragma unroll
@@ -183,22 +188,15 @@ __global__ void __launch_bounds__(NW * 64) stage1_mfma_kernel(const KernelParams
   // 32-column block; lane s of the group addresses key s/4, columns 4*(s%4) .. +3.
   const int v_rd = (4 * lh + (lane & 15) / 4) * SM::kVPitch + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
 
-  issue_loads(0);
-  for (int t = 0; t < ntiles; ++t) {
-    const int buf = t & 1;
-    store_lds(buf);
-    __syncthreads();
-    if (t + 1 < ntiles) issue_loads(t + 1);
-    if (!wave_active) continue;
-
-    const bool tree = t >= cache_tiles;
-    const int key0 = tree ? (t - cache_tiles) * kKeyTile : kv_start + t * kKeyTile;
-    const int key_lim = tree ? L : kv_end;
-    const bool masked = tree || (key0 + kKeyTile > key_lim);
+  // ---- one 64-key tile: S^T = K Q^T, online softmax, O^T += V^T P^T.
+  // MASKED tiles (the tree block, the ragged last cache tile) scale explicitly, add the
+  // mask, blank keys past the limit and run a second, compensating P.V product; full
+  // cache tiles take the lean path.
+  auto process_tile = [&](auto masked_c, int buf, bool tree, int key0, int key_lim) __attribute__((always_inline)) {
+    constexpr bool MASKED = decltype(masked_c)::value;
     const char* Kb = smem + buf * SM::kKBuf;
     const char* Vb = smem + 2 * SM::kKBuf + buf * SM::kVBuf;
 
-    // ---- S^T = K Q^T
     f32x16 s[2][QB];
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
@@ -206,23 +204,41 @@ __global__ void __launch_bounds__(NW * 64) stage1_mfma_kernel(const KernelParams
       for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[kb][qb][r] = 0.f;
+    {
+      // K fragments stream through a short register queue: kPF reads ahead of the MFMA
+      // that consumes them, so LDS latency hides under the matrix pipeline without
+      // holding the whole tile's fragments live.
+      constexpr int kFrags = 2 * KS;
+      constexpr int kPF = 4;
+      Vec8 kf[kFrags];
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const u32x4 raw = *reinterpret_cast<const u32x4*>(Kb + k_rd + kb * 32 * SM::kKPitch + ks * 32);
-        const Vec8 a = __builtin_bit_cast(Vec8, raw);
-#pragma unroll
-        for (int qb = 0; qb < QB; ++qb) s[kb][qb] = M::mma(a, qf[qb][ks], s[kb][qb]);
+      for (int f = 0; f < kFrags; ++f) {
+#ifdef FTA_DBG_NO_LDSREAD
+        const u32x4 raw = *reinterpret_cast<const u32x4*>(Kb + k_rd + (f & 1) * 32);
+#else
+        const u32x4 raw = *reinterpret_cast<const u32x4*>(Kb + k_rd + (f / KS) * 32 * SM::kKPitch + (f % KS) * 32);
+#endif
+        kf[f] = __builtin_bit_cast(Vec8, raw);
       }
+#pragma unroll
+      for (int f = 0; f < kFrags; ++f)
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) s[f / KS][qb] = M::mma(kf[f], qf[qb][f % KS], s[f / KS][qb]);
+      __builtin_amdgcn_sched_group_barrier(0x100, kPF, 0);
+#pragma unroll
+      for (int i = 0; i < kFrags - kPF; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, QB, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, kPF * QB, 0);
     }
 
-    // ---- online softmax; P^T packed to T in the B-operand layout of the PV product
+    // online softmax; P^T packed to T in the B-operand layout of the P.V product
     Vec8 pf[QB][4];
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
-      float m_old = m_run[qb], m_new, m_use;
-      if (masked) {
+      const float m_old = m_run[qb];
+      if (MASKED) {
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -234,25 +250,33 @@ __global__ void __launch_bounds__(NW * 64) stage1_mfma_kernel(const KernelParams
             s[kb][qb][r] = j < key_lim ? sv : neg_inf();
           }
       }
-      float mx = neg_inf();
+      float mx0 = fmaxf(s[0][qb][0], s[1][qb][0]), mx1 = fmaxf(s[0][qb][1], s[1][qb][1]);
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[kb][qb][r]);
-      mx = half_swap_max(mx, lh);
-      m_new = fmaxf(m_old, masked ? mx : mx * c);
-      m_use = (m_new == neg_inf()) ? 0.f : m_new;
+      for (int r = 2; r < 16; r += 2) {
+        mx0 = fmaxf(mx0, fmaxf(s[0][qb][r], s[1][qb][r]));
+        mx1 = fmaxf(mx1, fmaxf(s[0][qb][r + 1], s[1][qb][r + 1]));
+      }
+      const float mx = half_swap_max(fmaxf(mx0, mx1), lh);
+      const float m_new = fmaxf(m_old, MASKED ? mx : mx * c);
+      const float m_use = (MASKED && m_new == neg_inf()) ? 0.f : m_new;
       const float alpha = fast_exp2(m_old - m_use);
-      float psum = 0.f;
+      float ps0 = 0.f, ps1 = 0.f;
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float pv = masked ? fast_exp2(s[kb][qb][r] - m_use) : fast_exp2(__builtin_fmaf(s[kb][qb][r], c, -m_use));
-          s[kb][qb][r] = pv;
-          psum += pv;
+        for (int r = 0; r < 16; r += 2) {
+#ifdef FTA_DBG_NO_EXP
+          const float p0 = __builtin_fmaf(s[kb][qb][r], c, -m_use), p1 = __builtin_fmaf(s[kb][qb][r + 1], c, -m_use);
+#else
+          const float p0 = MASKED ? fast_exp2(s[kb][qb][r] - m_use) : fast_exp2(__builtin_fmaf(s[kb][qb][r], c, -m_use));
+          const float p1 = MASKED ? fast_exp2(s[kb][qb][r + 1] - m_use) : fast_exp2(__builtin_fmaf(s[kb][qb][r + 1], c, -m_use));
+#endif
+          s[kb][qb][r] = p0;
+          s[kb][qb][r + 1] = p1;
+          ps0 += p0;
+          ps1 += p1;
         }
-      l_run[qb] = l_run[qb] * alpha + psum;
+      l_run[qb] = l_run[qb] * alpha + (ps0 + ps1);
       m_run[qb] = m_new;
       if (__builtin_amdgcn_ballot_w64(m_new > m_old) != 0) {
 #pragma unroll
@@ -264,23 +288,30 @@ __global__ void __launch_bounds__(NW * 64) stage1_mfma_kernel(const KernelParams
       for (int kk = 0; kk < 4; ++kk) {
         Vec8 pk;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const float pv = s[kk >> 1][qb][(kk & 1) * 8 + e];
-          pk[e] = static_cast<T>(pv);
-          // masked tiles keep the rounding residue for a second, compensating product
-          if (masked) s[kk >> 1][qb][(kk & 1) * 8 + e] = pv - static_cast<float>(pk[e]);
+        for (int e = 0; e < 8; e += 2) {
+          const f32x2 pv = {s[kk >> 1][qb][(kk & 1) * 8 + e], s[kk >> 1][qb][(kk & 1) * 8 + e + 1]};
+          const auto pr = __builtin_convertvector(pv, typename M::Vec2);
+          pk[e] = pr[0];
+          pk[e + 1] = pr[1];
+          if (MASKED) {  // keep the rounding residue for the compensating product
+            s[kk >> 1][qb][(kk & 1) * 8 + e] = pv[0] - static_cast<float>(pr[0]);
+            s[kk >> 1][qb][(kk & 1) * 8 + e + 1] = pv[1] - static_cast<float>(pr[1]);
+          }
         }
         pf[qb][kk] = pk;
       }
     }
 
-    // ---- O^T += V^T P^T
-    auto pv_product = [&]() {
+    auto pv_product = [&]() __attribute__((always_inline)) {
 #pragma unroll
       for (int kk = 0; kk < 4; ++kk) {
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
+#ifdef FTA_DBG_NO_LDSREAD
+          const char* va = Vb + v_rd + (kk & 1) * 16 * SM::kVPitch;
+#else
           const char* va = Vb + v_rd + (kk * 16) * SM::kVPitch + db * 64;
+#endif
           const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 FTA_LDS*)(va));
           const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 FTA_LDS*)(va + 8 * SM::kVPitch));
           const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
@@ -290,8 +321,10 @@ __global__ void __launch_bounds__(NW * 64) stage1_mfma_kernel(const KernelParams
         }
       }
     };
+#ifndef FTA_DBG_NO_PV
     pv_product();
-    if (masked) {
+#endif
+    if (MASKED) {
       // Tree tiles and the ragged last cache tile are where single keys can carry large
       // weights (short sequences); a second product with the low-order part of P removes
       // the 2^-9 rounding of P there. Full cache tiles use one product.
@@ -306,6 +339,34 @@ __global__ void __launch_bounds__(NW * 64) stage1_mfma_kernel(const KernelParams
         }
       pv_product();
     }
+  };
+
+  // Two loops over one software pipeline: full cache tiles take the lean body, the
+  // ragged last cache tile and the tree tiles the masked one. Tile t+1 is in flight
+  // (global -> registers) while tile t is consumed from LDS.
+  const int full_tiles = kv_end > kv_start ? (kv_end - kv_start) / kKeyTile : 0;
+  issue_loads(0);
+  int t = 0;
+  for (; t < full_tiles; ++t) {
+#ifdef FTA_DBG_NO_GLOBAL
+    if (t == 0) { store_lds(0); store_lds(1); }
+    __syncthreads();
+#else
+    store_lds(t & 1);
+#ifndef FTA_DBG_NO_BARRIER
+    __syncthreads();
+#endif
+    if (t + 1 < ntiles) issue_loads(t + 1);
+#endif
+    if (wave_active) process_tile(std::false_type{}, t & 1, false, kv_start + t * kKeyTile, kv_end);
+  }
+  for (; t < ntiles; ++t) {
+    store_lds(t & 1);
+    __syncthreads();
+    if (t + 1 < ntiles) issue_loads(t + 1);
+    const bool tree = t >= cache_tiles;
+    const int key0 = tree ? (t - cache_tiles) * kKeyTile : kv_start + t * kKeyTile;
+    if (wave_active) process_tile(std::true_type{}, t & 1, tree, key0, tree ? L : kv_end);
   }
 
   if (!wave_active) return;
@@ -366,8 +427,8 @@ int launch(const KernelParams& p, hipStream_t stream) {
 template <typename T>
 int launch_t(const KernelParams& p, int head_dim, hipStream_t stream) {
   if (p.rows_per_wg == 256) {
-    if (head_dim == 128) return launch<T, 128, 2, 4>(p, stream);
-    if (head_dim == 64) return launch<T, 64, 2, 4>(p, stream);
+    if (head_dim == 128) return launch<T, 128, 1, 8>(p, stream);
+    if (head_dim == 64) return launch<T, 64, 1, 8>(p, stream);
   } else if (p.rows_per_wg == 128) {
     if (head_dim == 128) return launch<T, 128, 1, 4>(p, stream);
     if (head_dim == 64) return launch<T, 64, 1, 4>(p, stream);
