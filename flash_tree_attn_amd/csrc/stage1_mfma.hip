@@ -3,7 +3,9 @@
 // One workgroup = (batch, unit, split, row block). A unit is the set of query heads
 // that share one cache head (the GQA group) and one tree head, so its
 // rows = heads * q_len query rows all read the same K/V stream: every 64-key tile
-// of K and V is fetched from HBM once, staged in LDS, and consumed by all waves.
+// of K and V is fetched from HBM once, written straight into LDS by the load
+// instruction itself (global_load_lds, no register staging) into a ring of NS stages,
+// and consumed by all waves of the workgroup.
 //
 // Each wave owns QB blocks of 32 query rows and computes, per tile,
 //     S^T = K Q^T      (v_mfma_f32_32x32x16: A = K rows from LDS, B = Q in registers)
@@ -13,6 +15,14 @@
 // In the 32x32 accumulator layout lane (i, h) holds query row i and keys
 // 8*(r/4) + 4*h + r%4, r = 0..15; the same lane therefore already holds the B operand
 // of the second product if V^T's k-slots are read in that key order.
+//
+// LDS layout of one K or V tile (64 keys): blocks of RPB = 512/D rows, 1024 bytes each,
+// block pitch 1024 + pad. Inside a block the 16-byte chunks of its rows are interleaved
+// (chunk c of row r sits at c*16*RPB + r*16), which is what one wave-wide
+// global_load_lds writes when lane i fetches chunk i/RPB of row i%RPB. Both operand
+// read patterns (16 consecutive K rows at one chunk; 4 consecutive V rows x 64 bytes
+// for the transposing read) then fall on distinct banks, and every fragment address is
+// a per-lane base plus a compile-time offset.
 //
 // The split that owns the end of the sequence appends the tree block as extra tiles
 // (current_k / current_v with the additive mask), which replaces the eager block and
@@ -46,13 +56,21 @@ template <> struct Mfma<_Float16> {
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(8))) short s16x8;
 
+#define FTA_GLOBAL __attribute__((address_space(1)))
+
 template <int D>
-struct MfmaSmem {
-  static constexpr int kKPitch = D * 2 + 16;  // bytes; +16 keeps row-per-lane 128-bit reads conflict free
-  static constexpr int kVPitch = D * 2 + 64;  // bytes; +64 spreads the 4 key rows of a transposing read over all banks
-  static constexpr int kKBuf = kKeyTile * kKPitch;
-  static constexpr int kVBuf = kKeyTile * kVPitch;
-  static constexpr int kTotal = 2 * (kKBuf + kVBuf);
+struct TileLayout {
+  static constexpr int kRowBytes = D * 2;
+  static constexpr int kRowsPerBlock = 1024 / kRowBytes;           // 4 (D=128) or 8 (D=64)
+  static constexpr int kChunkStride = 16 * kRowsPerBlock;          // bytes between chunks of one row
+  static constexpr int kBlockPitch = 1024 + kChunkStride;          // pad: consecutive blocks shift banks
+  static constexpr int kBlocks = kKeyTile / kRowsPerBlock;         // 16 or 8
+  static constexpr int kTileBytes = kBlocks * kBlockPitch;
+  static constexpr int kStageBytes = 2 * kTileBytes;               // K tile then V tile
+  // byte offset of 16-byte chunk `c` of tile row `r`
+  static __device__ __forceinline__ int at(int r, int c) {
+    return (r / kRowsPerBlock) * kBlockPitch + c * kChunkStride + (r % kRowsPerBlock) * 16;
+  }
 };
 
 // Lanes i and i+32 hold the same query row. v_permlane32_swap exchanges the upper half
@@ -66,23 +84,73 @@ __device__ __forceinline__ float half_partner(float x, int lh) {
 __device__ __forceinline__ float half_swap_max(float x, int lh) { return fmaxf(x, half_partner(x, lh)); }
 __device__ __forceinline__ float half_swap_sum(float x, int lh) { return x + half_partner(x, lh); }
 
-template <typename T, int D, int QB, int NW>
+// s_waitcnt vmcnt(N) only (expcnt / lgkmcnt left at "no wait"), gfx9 encoding.
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt range");
+  __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4) | (0xF << 8));
+}
+
+// Operand fragments are read from LDS with explicit instructions and explicit
+// lgkmcnt waits. The compiler's own wait insertion treats every LDS read as possibly
+// aliasing the in-flight global_load_lds writes of LATER tiles and would drain them
+// (vmcnt 0) before each tile's reads, which defeats the multi-stage ring; reads it
+// cannot see are not subject to that. LDS returns data in issue order, so
+// "lgkmcnt <= N" means all but the N youngest reads have landed. The waited-for
+// registers are threaded through the wait so that their consumers cannot move above it.
+template <int OFF>
+__device__ __forceinline__ u32x4 lds_read_b128(uint32_t addr) {
+  u32x4 v;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+  return v;
+}
+template <int OFF>
+__device__ __forceinline__ u32x2 lds_read_tr16_b64(uint32_t addr) {
+  u32x2 v;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+  return v;
+}
+template <int N>
+__device__ __forceinline__ void wait_lgkm(u32x4& a) {
+  asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(a) : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void wait_lgkm(u32x2& a, u32x2& b) {
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
+}
+
+// Compile-time loop: f(std::integral_constant<int, I>) for I in [0, N).
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
+}
+
+template <typename T, int D, int QB, int NW, int NS>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(QB == 1 ? 2 : 1, QB == 1 ? 2 : 1)))
 stage1_mfma_kernel(const KernelParams p) {
   using M = Mfma<T>;
   using Vec8 = typename M::Vec8;
-  using SM = MfmaSmem<D>;
-  constexpr int kThreads = NW * 64;
+  using TL = TileLayout<D>;
   constexpr int KS = D / 16;                         // k-steps of the QK product
   constexpr int DB = D / 32;                         // head_dim blocks of the PV product
-  constexpr int kChunks = D / 8;                     // 16-byte chunks per row
-  constexpr int kRowsPerPass = kThreads / kChunks;   // rows one pass of the loader covers
-  constexpr int kPasses = kKeyTile / kRowsPerPass;
-  static_assert(kKeyTile % kRowsPerPass == 0 && kPasses >= 1, "loader mapping");
+  constexpr int RPB = TL::kRowsPerBlock;
+  constexpr int kLoadsPerTensor = TL::kBlocks / NW;  // global_load_lds per wave per tile, per K or V
+  static_assert(TL::kBlocks % NW == 0 && kLoadsPerTensor >= 1, "loader mapping");
+  constexpr int kLoadsPerTile = 2 * kLoadsPerTensor;
   constexpr int kRowsPerWave = 32 * QB;
   constexpr int kRowsPerWg = NW * kRowsPerWave;
 
   extern __shared__ __attribute__((aligned(16))) char smem[];
+#ifdef FTA_DBG_TIMING
+  long long dbg_t[12]; int dbg_n = 0; const long long dbg_c0 = clock64();
+#define FTA_STAMP() do { if (dbg_n < 12) dbg_t[dbg_n++] = wall_clock64(); } while (0)
+#else
+#define FTA_STAMP() do {} while (0)
+#endif
+  FTA_STAMP();
 
   const WorkItem w = decode_work(p, blockIdx.x);
   const int b = w.batch;
@@ -96,7 +164,7 @@ stage1_mfma_kernel(const KernelParams p) {
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int li = lane & 31;   // query row within a 32-row block / K row / V^T row
   const int lh = lane >> 5;   // half-wave: selects the k-slot group
   const int L = p.q_len;
@@ -107,10 +175,10 @@ stage1_mfma_kernel(const KernelParams p) {
   const bool wave_active = wave_row0 < p.rows;
   const float c = p.scale_log2;
 
-  const T* kbase = static_cast<const T*>(p.k) + b * p.k_stride[0] + cache_head * p.k_stride[1];
-  const T* vbase = static_cast<const T*>(p.v) + b * p.v_stride[0] + cache_head * p.v_stride[1];
-  const T* ckbase = static_cast<const T*>(p.ck) + b * p.ck_stride[0] + cur_head * p.ck_stride[1];
-  const T* cvbase = static_cast<const T*>(p.cv) + b * p.cv_stride[0] + cur_head * p.cv_stride[1];
+  const char* kbase = reinterpret_cast<const char*>(static_cast<const T*>(p.k) + b * p.k_stride[0] + cache_head * p.k_stride[1]);
+  const char* vbase = reinterpret_cast<const char*>(static_cast<const T*>(p.v) + b * p.v_stride[0] + cache_head * p.v_stride[1]);
+  const char* ckbase = reinterpret_cast<const char*>(static_cast<const T*>(p.ck) + b * p.ck_stride[0] + cur_head * p.ck_stride[1]);
+  const char* cvbase = reinterpret_cast<const char*>(static_cast<const T*>(p.cv) + b * p.cv_stride[0] + cur_head * p.cv_stride[1]);
 
   // ---- Q fragments (B operand of S^T = K Q^T), kept in registers for the whole split
   Vec8 qf[QB][KS];
@@ -131,6 +199,13 @@ stage1_mfma_kernel(const KernelParams p) {
     }
   }
 
+  // Q must have landed before the tile loop: a pending register load inside the loop
+  // would make the compiler drain ALL vector-memory traffic (vmcnt 0) every iteration,
+  // including the K/V tiles that are meant to stay in flight.
+  FTA_STAMP();
+  wait_vmcnt<0>();
+  FTA_STAMP();
+
   f32x16 o[DB][QB];
   float m_run[QB], l_run[QB];
 #pragma unroll
@@ -144,59 +219,71 @@ stage1_mfma_kernel(const KernelParams p) {
   }
 
   const int cache_tiles = kv_end > kv_start ? (kv_end - kv_start + kKeyTile - 1) / kKeyTile : 0;
+  const int full_tiles = kv_end > kv_start ? (kv_end - kv_start) / kKeyTile : 0;
   const int tree_tiles = owns_tree ? (L + kKeyTile - 1) / kKeyTile : 0;
   const int ntiles = cache_tiles + tree_tiles;
 
-  // ---- global -> register staging of one K/V tile
-  const int ld_row = tid / kChunks;
-  const int ld_chunk = tid % kChunks;
-  u32x4 kreg[kPasses], vreg[kPasses];
-  auto issue_loads = [&](int t) __attribute__((always_inline)) {
+  // ---- HBM -> LDS: lane i of a wave-wide load fetches chunk i/RPB of row i%RPB of one
+  // block; the hardware writes lane i's 16 bytes at block_base + 16*i.
+  const int ld_rib = lane % RPB;
+  const int ld_chunk = lane / RPB;
+  const uint32_t k_lane_off = static_cast<uint32_t>(ld_rib * p.k_stride[2] * 2 + ld_chunk * 16);
+  const uint32_t v_lane_off = static_cast<uint32_t>(ld_rib * p.v_stride[2] * 2 + ld_chunk * 16);
+  const int64_t k_row_bytes = p.k_stride[2] * 2, v_row_bytes = p.v_stride[2] * 2;
+
+  auto issue_full_tile = [&](int t) __attribute__((always_inline)) {
+    char* stage = smem + (t % NS) * TL::kStageBytes;
+    const int key0 = kv_start + t * kKeyTile;
+#pragma unroll
+    for (int i = 0; i < kLoadsPerTensor; ++i) {
+      const int blk = i * NW + wave;
+      const char* ksrc = kbase + static_cast<int64_t>(key0 + blk * RPB) * k_row_bytes;
+      const char* vsrc = vbase + static_cast<int64_t>(key0 + blk * RPB) * v_row_bytes;
+      __builtin_amdgcn_global_load_lds((const FTA_GLOBAL void*)(ksrc + k_lane_off), (FTA_LDS void*)(stage + blk * TL::kBlockPitch), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const FTA_GLOBAL void*)(vsrc + v_lane_off),
+                                       (FTA_LDS void*)(stage + TL::kTileBytes + blk * TL::kBlockPitch), 16, 0, 0);
+    }
+  };
+  // Ragged / tree tiles: rows past the limit re-read the last valid row (finite data
+  // that the -inf logits then ignore) instead of touching padding.
+  auto issue_edge_tile = [&](int t) __attribute__((always_inline)) {
+    char* stage = smem + (t % NS) * TL::kStageBytes;
     const bool tree = t >= cache_tiles;
     const int key0 = tree ? (t - cache_tiles) * kKeyTile : kv_start + t * kKeyTile;
     const int key_lim = tree ? L : kv_end;
-    const T* kb_ = tree ? ckbase : kbase;
-    const T* vb_ = tree ? cvbase : vbase;
-    const int64_t kts = tree ? p.ck_stride[2] : p.k_stride[2];
-    const int64_t vts = tree ? p.cv_stride[2] : p.v_stride[2];
+    const char* kb_ = tree ? ckbase : kbase;
+    const char* vb_ = tree ? cvbase : vbase;
+    const int64_t krb = tree ? p.ck_stride[2] * 2 : k_row_bytes;
+    const int64_t vrb = tree ? p.cv_stride[2] * 2 : v_row_bytes;
 #pragma unroll
-    for (int ps = 0; ps < kPasses; ++ps) {
-      const int j = key0 + ps * kRowsPerPass + ld_row;
-      u32x4 kq = {0, 0, 0, 0}, vq = {0, 0, 0, 0};
-      if (j < key_lim) {
-        kq = *reinterpret_cast<const u32x4*>(kb_ + j * kts + ld_chunk * 8);
-        vq = *reinterpret_cast<const u32x4*>(vb_ + j * vts + ld_chunk * 8);
-      }
-      kreg[ps] = kq;
-      vreg[ps] = vq;
+    for (int i = 0; i < kLoadsPerTensor; ++i) {
+      const int blk = i * NW + wave;
+      const int j = min(key0 + blk * RPB + ld_rib, key_lim - 1);
+      __builtin_amdgcn_global_load_lds((const FTA_GLOBAL void*)(kb_ + j * krb + ld_chunk * 16), (FTA_LDS void*)(stage + blk * TL::kBlockPitch), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const FTA_GLOBAL void*)(vb_ + j * vrb + ld_chunk * 16),
+                                       (FTA_LDS void*)(stage + TL::kTileBytes + blk * TL::kBlockPitch), 16, 0, 0);
     }
   };
-  auto store_lds = [&](int buf) __attribute__((always_inline)) {
-    char* kdst = smem + buf * SM::kKBuf;
-    char* vdst = smem + 2 * SM::kKBuf + buf * SM::kVBuf;
-#pragma unroll
-    for (int ps = 0; ps < kPasses; ++ps) {
-      const int j = ps * kRowsPerPass + ld_row;
-      *reinterpret_cast<u32x4*>(kdst + j * SM::kKPitch + ld_chunk * 16) = kreg[ps];
-      *reinterpret_cast<u32x4*>(vdst + j * SM::kVPitch + ld_chunk * 16) = vreg[ps];
-    }
+  auto issue_tile = [&](int t) __attribute__((always_inline)) {
+    if (t < full_tiles) issue_full_tile(t); else issue_edge_tile(t);
   };
 
-  // per-lane LDS byte offsets of the operand reads
-  const int k_rd = li * SM::kKPitch + lh * 16;  // + kb*32*pitch + ks*32
+  // per-lane LDS byte offsets of the operand reads (everything else is a constant)
+  const uint32_t smem_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((FTA_LDS char*)smem));
+  const int k_rd = smem_base + TL::at(li, lh);                       // + kb * (32/RPB) * pitch + ks * 2 * chunk stride
   // V^T transposing read: 16-lane group g covers head_dim columns 16*(g%2) .. +15 of a
   // 32-column block; lane s of the group addresses key s/4, columns 4*(s%4) .. +3.
-  const int v_rd = (4 * lh + (lane & 15) / 4) * SM::kVPitch + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+  const int v_rd = smem_base + TL::at(4 * lh + (lane & 15) / 4, 2 * ((lane >> 4) & 1) + ((lane >> 1) & 1)) + (lane & 1) * 8;
+  // + (16*kk + 8*hi rows) + db * 4 chunks
+  constexpr int kVRowsOff8 = (8 / RPB) * TL::kBlockPitch + (8 % RPB) * 16;    // 8 rows further
+  constexpr int kVRowsOff16 = (16 / RPB) * TL::kBlockPitch;                   // 16 rows further
 
   // ---- one 64-key tile: S^T = K Q^T, online softmax, O^T += V^T P^T.
   // MASKED tiles (the tree block, the ragged last cache tile) scale explicitly, add the
   // mask, blank keys past the limit and run a second, compensating P.V product; full
   // cache tiles take the lean path.
-  auto process_tile = [&](auto masked_c, int buf, bool tree, int key0, int key_lim) __attribute__((always_inline)) {
+  auto process_tile = [&](auto masked_c, int stage_idx, bool tree, int key0, int key_lim) __attribute__((always_inline)) {
     constexpr bool MASKED = decltype(masked_c)::value;
-    const char* Kb = smem + buf * SM::kKBuf;
-    const char* Vb = smem + 2 * SM::kKBuf + buf * SM::kVBuf;
-
     f32x16 s[2][QB];
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
@@ -206,32 +293,36 @@ stage1_mfma_kernel(const KernelParams p) {
         for (int r = 0; r < 16; ++r) s[kb][qb][r] = 0.f;
     {
       // K fragments stream through a short register queue: kPF reads ahead of the MFMA
-      // that consumes them, so LDS latency hides under the matrix pipeline without
-      // holding the whole tile's fragments live.
+      // that consumes them, so LDS latency hides under the matrix pipeline.
       constexpr int kFrags = 2 * KS;
       constexpr int kPF = 4;
-      Vec8 kf[kFrags];
+      constexpr int kKbOff = (32 / RPB) * TL::kBlockPitch, kKsOff = 2 * TL::kChunkStride;
+      const uint32_t ka = static_cast<uint32_t>(k_rd + stage_idx * TL::kStageBytes);
+      u32x4 kf[kFrags];
+      static_for<0, kPF>([&](auto f) { kf[f] = lds_read_b128<(f / KS) * kKbOff + (f % KS) * kKsOff>(ka); });
+      static_for<0, kFrags>([&](auto f) {
+        constexpr int kNewer = (kFrags - 1 - f) < (kPF - 1) ? (kFrags - 1 - f) : (kPF - 1);
+        wait_lgkm<kNewer>(kf[f]);
+        const Vec8 a = __builtin_bit_cast(Vec8, kf[f]);
 #pragma unroll
-      for (int f = 0; f < kFrags; ++f) {
-#ifdef FTA_DBG_NO_LDSREAD
-        const u32x4 raw = *reinterpret_cast<const u32x4*>(Kb + k_rd + (f & 1) * 32);
-#else
-        const u32x4 raw = *reinterpret_cast<const u32x4*>(Kb + k_rd + (f / KS) * 32 * SM::kKPitch + (f % KS) * 32);
-#endif
-        kf[f] = __builtin_bit_cast(Vec8, raw);
-      }
-#pragma unroll
-      for (int f = 0; f < kFrags; ++f)
-#pragma unroll
-        for (int qb = 0; qb < QB; ++qb) s[f / KS][qb] = M::mma(kf[f], qf[qb][f % KS], s[f / KS][qb]);
-      __builtin_amdgcn_sched_group_barrier(0x100, kPF, 0);
-#pragma unroll
-      for (int i = 0; i < kFrags - kPF; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, QB, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      }
-      __builtin_amdgcn_sched_group_barrier(0x008, kPF * QB, 0);
+        for (int qb = 0; qb < QB; ++qb) s[f / KS][qb] = M::mma(a, qf[qb][f % KS], s[f / KS][qb]);
+        if constexpr (f + kPF < kFrags)
+          kf[f + kPF] = lds_read_b128<((f + kPF) / KS) * kKbOff + ((f + kPF) % KS) * kKsOff>(ka);
+      });
     }
+
+    // V^T fragment queue (two transposing reads per fragment); the first kVPF fragments
+    // are requested now so that their latency hides under the softmax.
+    constexpr int kVFrags = 4 * DB;
+    constexpr int kVPF = 4;
+    const uint32_t va = static_cast<uint32_t>(v_rd + stage_idx * TL::kStageBytes + TL::kTileBytes);
+    u32x2 vlo[kVFrags], vhi[kVFrags];
+    auto issue_v = [&](auto g) __attribute__((always_inline)) {
+      constexpr int kOff = (g / DB) * kVRowsOff16 + (g % DB) * 4 * TL::kChunkStride;
+      vlo[g] = lds_read_tr16_b64<kOff>(va);
+      vhi[g] = lds_read_tr16_b64<kOff + kVRowsOff8>(va);
+    };
+    static_for<0, kVPF>(issue_v);
 
     // online softmax; P^T packed to T in the B-operand layout of the P.V product
     Vec8 pf[QB][4];
@@ -239,14 +330,26 @@ stage1_mfma_kernel(const KernelParams p) {
     for (int qb = 0; qb < QB; ++qb) {
       const float m_old = m_run[qb];
       if (MASKED) {
+        // Mask values are fetched with clamped indices and no branches, so that all of a
+        // tile's loads are in flight together (one memory round trip, not one per value).
+        float mv[2][16];
+        if (tree) {
+          const float* mrow = p.mask + b * p.mask_stride[0] + row_head[qb] * p.mask_stride[1] + row_i[qb] * p.mask_stride[2];
+#pragma unroll
+          for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int j = key0 + kb * 32 + (r >> 2) * 8 + 4 * lh + (r & 3);
+              mv[kb][r] = mrow[min(j, key_lim - 1)];
+            }
+        }
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             const int j = key0 + kb * 32 + (r >> 2) * 8 + 4 * lh + (r & 3);
             float sv = s[kb][qb][r] * c;
-            if (tree && j < key_lim && row_ok[qb])
-              sv += p.mask[b * p.mask_stride[0] + row_head[qb] * p.mask_stride[1] + row_i[qb] * p.mask_stride[2] + j] * kLog2e;
+            if (tree) sv = __builtin_fmaf(mv[kb][r], kLog2e, sv);
             s[kb][qb][r] = j < key_lim ? sv : neg_inf();
           }
       }
@@ -303,27 +406,17 @@ stage1_mfma_kernel(const KernelParams p) {
     }
 
     auto pv_product = [&]() __attribute__((always_inline)) {
+      static_for<0, kVFrags>([&](auto g) {
+        constexpr int kNewer = (kVFrags - 1 - g) < (kVPF - 1) ? (kVFrags - 1 - g) : (kVPF - 1);
+        wait_lgkm<2 * kNewer>(vlo[g], vhi[g]);
+        const s16x8 both = __builtin_shufflevector(__builtin_bit_cast(s16x4, vlo[g]), __builtin_bit_cast(s16x4, vhi[g]), 0, 1, 2, 3, 4, 5, 6, 7);
+        const Vec8 a = __builtin_bit_cast(Vec8, both);
 #pragma unroll
-      for (int kk = 0; kk < 4; ++kk) {
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-#ifdef FTA_DBG_NO_LDSREAD
-          const char* va = Vb + v_rd + (kk & 1) * 16 * SM::kVPitch;
-#else
-          const char* va = Vb + v_rd + (kk * 16) * SM::kVPitch + db * 64;
-#endif
-          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 FTA_LDS*)(va));
-          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 FTA_LDS*)(va + 8 * SM::kVPitch));
-          const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-          const Vec8 a = __builtin_bit_cast(Vec8, both);
-#pragma unroll
-          for (int qb = 0; qb < QB; ++qb) o[db][qb] = M::mma(a, pf[qb][kk], o[db][qb]);
-        }
-      }
+        for (int qb = 0; qb < QB; ++qb) o[g % DB][qb] = M::mma(a, pf[qb][g / DB], o[g % DB][qb]);
+        if constexpr (g + kVPF < kVFrags) issue_v(std::integral_constant<int, g + kVPF>{});
+      });
     };
-#ifndef FTA_DBG_NO_PV
     pv_product();
-#endif
     if (MASKED) {
       // Tree tiles and the ragged last cache tile are where single keys can carry large
       // weights (short sequences); a second product with the low-order part of P removes
@@ -337,38 +430,58 @@ stage1_mfma_kernel(const KernelParams p) {
           for (int e = 0; e < 8; ++e) pk[e] = static_cast<T>(s[kk >> 1][qb][(kk & 1) * 8 + e]);
           pf[qb][kk] = pk;
         }
+      static_for<0, kVPF>(issue_v);
       pv_product();
     }
   };
 
-  // Two loops over one software pipeline: full cache tiles take the lean body, the
-  // ragged last cache tile and the tree tiles the masked one. Tile t+1 is in flight
-  // (global -> registers) while tile t is consumed from LDS.
-  const int full_tiles = kv_end > kv_start ? (kv_end - kv_start) / kKeyTile : 0;
-  issue_loads(0);
+  // ---- the pipeline: tiles t+1 .. t+NS-1 are in flight (HBM -> LDS) while tile t is
+  // consumed. Per tile: wait until this wave's share of tile t has landed, barrier
+  // (everybody's share has landed AND everybody is done with tile t-1, whose stage is
+  // the one the next load reuses), issue tile t+NS-1, compute tile t.
+#pragma unroll
+  for (int t = 0; t < NS - 1; ++t)
+    if (t < ntiles) issue_tile(t);
+
+  auto wait_tile = [&](int t) __attribute__((always_inline)) {
+    // loads issued after tile t's: min(NS-2, ntiles-1-t) tiles of kLoadsPerTile each
+    const int ahead = min(NS - 2, ntiles - 1 - t);
+    if (NS >= 4 && ahead >= 2) wait_vmcnt<2 * kLoadsPerTile>();
+    else if (NS >= 3 && ahead >= 1) wait_vmcnt<kLoadsPerTile>();
+    else wait_vmcnt<0>();
+  };
+
+  FTA_STAMP();
   int t = 0;
   for (; t < full_tiles; ++t) {
 #ifdef FTA_DBG_NO_GLOBAL
-    if (t == 0) { store_lds(0); store_lds(1); }
-    __syncthreads();
-#else
-    store_lds(t & 1);
+    wait_vmcnt<0>();
 #ifndef FTA_DBG_NO_BARRIER
-    __syncthreads();
+    __builtin_amdgcn_s_barrier();
 #endif
-    if (t + 1 < ntiles) issue_loads(t + 1);
+#else
+    wait_tile(t);
+#ifndef FTA_DBG_NO_BARRIER
+    __builtin_amdgcn_s_barrier();
 #endif
-    if (wave_active) process_tile(std::false_type{}, t & 1, false, kv_start + t * kKeyTile, kv_end);
+    if (t + NS - 1 < ntiles) issue_tile(t + NS - 1);
+#endif
+#ifndef FTA_DBG_NO_COMPUTE
+    if (wave_active) process_tile(std::false_type{}, t % NS, false, kv_start + t * kKeyTile, kv_end);
+#endif
   }
+  FTA_STAMP();
   for (; t < ntiles; ++t) {
-    store_lds(t & 1);
-    __syncthreads();
-    if (t + 1 < ntiles) issue_loads(t + 1);
+    wait_tile(t);
+    FTA_STAMP();
+    __builtin_amdgcn_s_barrier();
+    if (t + NS - 1 < ntiles) issue_tile(t + NS - 1);
     const bool tree = t >= cache_tiles;
     const int key0 = tree ? (t - cache_tiles) * kKeyTile : kv_start + t * kKeyTile;
-    if (wave_active) process_tile(std::true_type{}, t & 1, tree, key0, tree ? L : kv_end);
+    if (wave_active) process_tile(std::true_type{}, t % NS, tree, key0, tree ? L : kv_end);
   }
 
+  FTA_STAMP();
   if (!wave_active) return;
 
   // ---- epilogue
@@ -407,31 +520,46 @@ stage1_mfma_kernel(const KernelParams p) {
       }
     }
   }
+#ifdef FTA_DBG_TIMING
+  FTA_STAMP();
+  if (tid == 0 && (blockIdx.x == 0 || blockIdx.x == 255)) {
+    long long* dst = reinterpret_cast<long long*>(p.mid_lse) + (blockIdx.x == 0 ? 0 : 16);
+    for (int i = 0; i < dbg_n; ++i) dst[i] = dbg_t[i];
+    dst[15] = dbg_n; dst[14] = clock64() - dbg_c0;
+  }
+#endif
 }
 
-template <typename T, int D, int QB, int NW>
+template <typename T, int D, int QB, int NW, int NS>
 int launch(const KernelParams& p, hipStream_t stream) {
-  using SM = MfmaSmem<D>;
-  auto kern = stage1_mfma_kernel<T, D, QB, NW>;
-  if (SM::kTotal > 64 * 1024) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            SM::kTotal) != hipSuccess)
-      return FTA_ERR_LAUNCH;
+  constexpr int kSmem = NS * TileLayout<D>::kStageBytes;
+  static_assert(kSmem <= 160 * 1024, "LDS budget");
+  auto kern = stage1_mfma_kernel<T, D, QB, NW, NS>;
+  if (kSmem > 64 * 1024) {
+    // Raising the dynamic-LDS limit is a driver call: once per kernel and device, not per launch.
+    static thread_local int configured_device = -1;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return FTA_ERR_NO_DEVICE;
+    if (configured_device != dev) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kSmem) != hipSuccess)
+        return FTA_ERR_LAUNCH;
+      configured_device = dev;
+    }
   }
   const int64_t grid = static_cast<int64_t>(p.bsz) * p.units * p.row_blocks * p.num_splits;
   if (grid <= 0 || grid > 0x7fffffffLL) return FTA_ERR_SHAPE;
-  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(grid)), dim3(NW * 64), SM::kTotal, stream, p);
+  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(grid)), dim3(NW * 64), kSmem, stream, p);
   return hipGetLastError() == hipSuccess ? FTA_OK : FTA_ERR_LAUNCH;
 }
 
 template <typename T>
 int launch_t(const KernelParams& p, int head_dim, hipStream_t stream) {
-  if (p.rows_per_wg == 256) {
-    if (head_dim == 128) return launch<T, 128, 1, 8>(p, stream);
-    if (head_dim == 64) return launch<T, 64, 1, 8>(p, stream);
-  } else if (p.rows_per_wg == 128) {
-    if (head_dim == 128) return launch<T, 128, 1, 4>(p, stream);
-    if (head_dim == 64) return launch<T, 64, 1, 4>(p, stream);
+  if (p.rows_per_wg == 256) {  // 8 waves, one workgroup per CU, 4-stage ring
+    if (head_dim == 128) return launch<T, 128, 1, 8, 4>(p, stream);
+    if (head_dim == 64) return launch<T, 64, 1, 8, 4>(p, stream);
+  } else if (p.rows_per_wg == 128) {  // 4 waves, two workgroups per CU, 2-stage ring each
+    if (head_dim == 128) return launch<T, 128, 1, 4, 2>(p, stream);
+    if (head_dim == 64) return launch<T, 64, 1, 4, 2>(p, stream);
   }
   return FTA_ERR_UNSUPPORTED;
 }
@@ -440,6 +568,8 @@ int launch_t(const KernelParams& p, int head_dim, hipStream_t stream) {
 
 int launch_stage1_mfma(const KernelParams& p, int dtype, int head_dim, void* stream) {
   if (p.scale_log2 <= 0.f) return FTA_ERR_UNSUPPORTED;  // row max is taken before scaling
+  // Loads address each K/V stream with 32-bit lane offsets.
+  if (p.k_stride[2] * 2 * 8 > 0x7fffffffLL || p.v_stride[2] * 2 * 8 > 0x7fffffffLL) return FTA_ERR_UNSUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (dtype) {
     case FTA_F16: return launch_t<_Float16>(p, head_dim, s);

@@ -205,9 +205,16 @@ int launch(const KernelParams& p, hipStream_t stream) {
   using S = ShuffleSmem<T, D>;
   auto kern = stage1_shuffle_kernel<T, D>;
   if (S::kTotal > 64 * 1024) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            S::kTotal) != hipSuccess)
-      return FTA_ERR_LAUNCH;
+    // Raising the dynamic-LDS limit is a driver call: once per kernel and device, not per launch.
+    static thread_local int configured_device = -1;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return FTA_ERR_NO_DEVICE;
+    if (configured_device != dev) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              S::kTotal) != hipSuccess)
+        return FTA_ERR_LAUNCH;
+      configured_device = dev;
+    }
   }
   const int64_t grid = static_cast<int64_t>(p.bsz) * p.units * p.row_blocks * p.num_splits;
   if (grid <= 0 || grid > 0x7fffffffLL) return FTA_ERR_SHAPE;
