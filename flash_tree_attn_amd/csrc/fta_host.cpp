@@ -83,7 +83,7 @@ int plan(const fta_args& a, int num_cus, fta_plan_out* out) {
   const int rows_per_wg = kernel == FTA_KERNEL_MFMA ? mfma_rows_per_wg(rows) : 16;
   const int row_blocks = static_cast<int>(cdiv(rows, rows_per_wg));
   // Workgroups one CU holds at a time (LDS- and register-bound, see the kernels).
-  const int wg_per_cu = kernel == FTA_KERNEL_MFMA ? (rows_per_wg == 256 ? 1 : 2) : 1;
+  const int wg_per_cu = 1;
 
   const int64_t work_items = static_cast<int64_t>(a.bsz) * units * row_blocks;
   const int64_t t_cap = a.max_seq_len_hint > 0 ? std::min(a.max_seq_len_hint, a.cache_len) : a.cache_len;

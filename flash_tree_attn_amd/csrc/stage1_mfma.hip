@@ -128,12 +128,16 @@ __device__ __forceinline__ void static_for(F&& f) {
   }
 }
 
-template <typename T, int D, int QB, int NW, int NS>
+// NSK >= 2: K of tile t+1 is read during iteration t and must have been requested an
+// iteration earlier.
+template <typename T, int D, int QB, int NW, int NSK>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(QB == 1 ? 2 : 1, QB == 1 ? 2 : 1)))
 stage1_mfma_kernel(const KernelParams p) {
   using M = Mfma<T>;
   using Vec8 = typename M::Vec8;
   using TL = TileLayout<D>;
+  static_assert(NSK >= 2, "K ring too shallow");
+  constexpr int NSV = NSK + 2;                       // V of a tile is read one iteration after its K
   constexpr int KS = D / 16;                         // k-steps of the QK product
   constexpr int DB = D / 32;                         // head_dim blocks of the PV product
   constexpr int RPB = TL::kRowsPerBlock;
@@ -142,15 +146,9 @@ stage1_mfma_kernel(const KernelParams p) {
   constexpr int kLoadsPerTile = 2 * kLoadsPerTensor;
   constexpr int kRowsPerWave = 32 * QB;
   constexpr int kRowsPerWg = NW * kRowsPerWave;
+  constexpr int kVRing = NSK * TL::kTileBytes;       // byte offset of the V ring
 
   extern __shared__ __attribute__((aligned(16))) char smem[];
-#ifdef FTA_DBG_TIMING
-  long long dbg_t[12]; int dbg_n = 0; const long long dbg_c0 = clock64();
-#define FTA_STAMP() do { if (dbg_n < 12) dbg_t[dbg_n++] = wall_clock64(); } while (0)
-#else
-#define FTA_STAMP() do {} while (0)
-#endif
-  FTA_STAMP();
 
   const WorkItem w = decode_work(p, blockIdx.x);
   const int b = w.batch;
@@ -180,6 +178,11 @@ stage1_mfma_kernel(const KernelParams p) {
   const char* ckbase = reinterpret_cast<const char*>(static_cast<const T*>(p.ck) + b * p.ck_stride[0] + cur_head * p.ck_stride[1]);
   const char* cvbase = reinterpret_cast<const char*>(static_cast<const T*>(p.cv) + b * p.cv_stride[0] + cur_head * p.cv_stride[1]);
 
+  const int cache_tiles = kv_end > kv_start ? (kv_end - kv_start + kKeyTile - 1) / kKeyTile : 0;
+  const int full_tiles = kv_end > kv_start ? (kv_end - kv_start) / kKeyTile : 0;
+  const int tree_tiles = owns_tree ? (L + kKeyTile - 1) / kKeyTile : 0;
+  const int ntiles = cache_tiles + tree_tiles;
+
   // ---- Q fragments (B operand of S^T = K Q^T), kept in registers for the whole split
   Vec8 qf[QB][KS];
   bool row_ok[QB];
@@ -199,32 +202,10 @@ stage1_mfma_kernel(const KernelParams p) {
     }
   }
 
-  // Q must have landed before the tile loop: a pending register load inside the loop
-  // would make the compiler drain ALL vector-memory traffic (vmcnt 0) every iteration,
-  // including the K/V tiles that are meant to stay in flight.
-  FTA_STAMP();
-  wait_vmcnt<0>();
-  FTA_STAMP();
-
-  f32x16 o[DB][QB];
-  float m_run[QB], l_run[QB];
-#pragma unroll
-  for (int qb = 0; qb < QB; ++qb) {
-    m_run[qb] = neg_inf();
-    l_run[qb] = 0.f;
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) o[db][qb][r] = 0.f;
-  }
-
-  const int cache_tiles = kv_end > kv_start ? (kv_end - kv_start + kKeyTile - 1) / kKeyTile : 0;
-  const int full_tiles = kv_end > kv_start ? (kv_end - kv_start) / kKeyTile : 0;
-  const int tree_tiles = owns_tree ? (L + kKeyTile - 1) / kKeyTile : 0;
-  const int ntiles = cache_tiles + tree_tiles;
-
   // ---- HBM -> LDS: lane i of a wave-wide load fetches chunk i/RPB of row i%RPB of one
-  // block; the hardware writes lane i's 16 bytes at block_base + 16*i.
+  // block; the hardware writes lane i's 16 bytes at block_base + 16*i. K tiles cycle
+  // through a ring of NSK stages, V tiles through NSV = NSK + 2 (V is consumed one
+  // iteration after K, see the pipeline below).
   const int ld_rib = lane % RPB;
   const int ld_chunk = lane / RPB;
   const uint32_t k_lane_off = static_cast<uint32_t>(ld_rib * p.k_stride[2] * 2 + ld_chunk * 16);
@@ -232,22 +213,23 @@ stage1_mfma_kernel(const KernelParams p) {
   const int64_t k_row_bytes = p.k_stride[2] * 2, v_row_bytes = p.v_stride[2] * 2;
 
   auto issue_full_tile = [&](int t) __attribute__((always_inline)) {
-    char* stage = smem + (t % NS) * TL::kStageBytes;
+    char* kst = smem + (t % NSK) * TL::kTileBytes;
+    char* vst = smem + kVRing + (t % NSV) * TL::kTileBytes;
     const int key0 = kv_start + t * kKeyTile;
 #pragma unroll
     for (int i = 0; i < kLoadsPerTensor; ++i) {
       const int blk = i * NW + wave;
       const char* ksrc = kbase + static_cast<int64_t>(key0 + blk * RPB) * k_row_bytes;
       const char* vsrc = vbase + static_cast<int64_t>(key0 + blk * RPB) * v_row_bytes;
-      __builtin_amdgcn_global_load_lds((const FTA_GLOBAL void*)(ksrc + k_lane_off), (FTA_LDS void*)(stage + blk * TL::kBlockPitch), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((const FTA_GLOBAL void*)(vsrc + v_lane_off),
-                                       (FTA_LDS void*)(stage + TL::kTileBytes + blk * TL::kBlockPitch), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const FTA_GLOBAL void*)(ksrc + k_lane_off), (FTA_LDS void*)(kst + blk * TL::kBlockPitch), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const FTA_GLOBAL void*)(vsrc + v_lane_off), (FTA_LDS void*)(vst + blk * TL::kBlockPitch), 16, 0, 0);
     }
   };
   // Ragged / tree tiles: rows past the limit re-read the last valid row (finite data
   // that the -inf logits then ignore) instead of touching padding.
   auto issue_edge_tile = [&](int t) __attribute__((always_inline)) {
-    char* stage = smem + (t % NS) * TL::kStageBytes;
+    char* kst = smem + (t % NSK) * TL::kTileBytes;
+    char* vst = smem + kVRing + (t % NSV) * TL::kTileBytes;
     const bool tree = t >= cache_tiles;
     const int key0 = tree ? (t - cache_tiles) * kKeyTile : kv_start + t * kKeyTile;
     const int key_lim = tree ? L : kv_end;
@@ -259,73 +241,150 @@ stage1_mfma_kernel(const KernelParams p) {
     for (int i = 0; i < kLoadsPerTensor; ++i) {
       const int blk = i * NW + wave;
       const int j = min(key0 + blk * RPB + ld_rib, key_lim - 1);
-      __builtin_amdgcn_global_load_lds((const FTA_GLOBAL void*)(kb_ + j * krb + ld_chunk * 16), (FTA_LDS void*)(stage + blk * TL::kBlockPitch), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((const FTA_GLOBAL void*)(vb_ + j * vrb + ld_chunk * 16),
-                                       (FTA_LDS void*)(stage + TL::kTileBytes + blk * TL::kBlockPitch), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const FTA_GLOBAL void*)(kb_ + j * krb + ld_chunk * 16), (FTA_LDS void*)(kst + blk * TL::kBlockPitch), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const FTA_GLOBAL void*)(vb_ + j * vrb + ld_chunk * 16), (FTA_LDS void*)(vst + blk * TL::kBlockPitch), 16, 0, 0);
     }
   };
   auto issue_tile = [&](int t) __attribute__((always_inline)) {
     if (t < full_tiles) issue_full_tile(t); else issue_edge_tile(t);
   };
 
-  // per-lane LDS byte offsets of the operand reads (everything else is a constant)
+  // Q must have landed before the tile loop: a pending register load inside the loop
+  // would make the compiler drain ALL vector-memory traffic (vmcnt 0) every iteration,
+  // including the K/V tiles that are meant to stay in flight. Then the first NSK tiles go out.
+  wait_vmcnt<0>();
+#pragma unroll
+  for (int t = 0; t < NSK; ++t)
+    if (t < ntiles) issue_tile(t);
+
+  f32x16 o[DB][QB];
+  float m_run[QB], l_run[QB], alpha_pending[QB];
+  bool rescale_pending = false;
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    m_run[qb] = neg_inf();
+    l_run[qb] = 0.f;
+    alpha_pending[qb] = 1.f;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[db][qb][r] = 0.f;
+  }
+
+  // per-lane LDS byte addresses of the operand reads (everything else is a constant)
   const uint32_t smem_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((FTA_LDS char*)smem));
-  const int k_rd = smem_base + TL::at(li, lh);                       // + kb * (32/RPB) * pitch + ks * 2 * chunk stride
+  const uint32_t k_rd = smem_base + TL::at(li, lh);  // + kb * (32/RPB) * pitch + ks * 2 * chunk stride
   // V^T transposing read: 16-lane group g covers head_dim columns 16*(g%2) .. +15 of a
   // 32-column block; lane s of the group addresses key s/4, columns 4*(s%4) .. +3.
-  const int v_rd = smem_base + TL::at(4 * lh + (lane & 15) / 4, 2 * ((lane >> 4) & 1) + ((lane >> 1) & 1)) + (lane & 1) * 8;
-  // + (16*kk + 8*hi rows) + db * 4 chunks
+  const uint32_t v_rd = smem_base + kVRing + TL::at(4 * lh + (lane & 15) / 4, 2 * ((lane >> 4) & 1) + ((lane >> 1) & 1)) + (lane & 1) * 8;
   constexpr int kVRowsOff8 = (8 / RPB) * TL::kBlockPitch + (8 % RPB) * 16;    // 8 rows further
   constexpr int kVRowsOff16 = (16 / RPB) * TL::kBlockPitch;                   // 16 rows further
+  constexpr int kKbOff = (32 / RPB) * TL::kBlockPitch, kKsOff = 2 * TL::kChunkStride;
+  constexpr int kKFrags = 2 * KS;   // K fragments per tile (one 128-bit read each)
+  constexpr int kVFrags = 4 * DB;   // V^T fragments per tile (two transposing reads each)
+  constexpr int kPF = 4;            // fragments requested ahead of the MFMA that consumes them
 
-  // ---- one 64-key tile: S^T = K Q^T, online softmax, O^T += V^T P^T.
-  // MASKED tiles (the tree block, the ragged last cache tile) scale explicitly, add the
-  // mask, blank keys past the limit and run a second, compensating P.V product; full
-  // cache tiles take the lean path.
-  auto process_tile = [&](auto masked_c, int stage_idx, bool tree, int key0, int key_lim) __attribute__((always_inline)) {
-    constexpr bool MASKED = decltype(masked_c)::value;
-    f32x16 s[2][QB];
+  // ---- building blocks -------------------------------------------------------------
+  // S^T = K Q^T of tile t (fragment queue: kPF reads ahead of the consuming MFMA).
+  auto qk_tile = [&](int t, f32x16 (&s)[2][QB]) __attribute__((always_inline)) {
+    const uint32_t ka = k_rd + (t % NSK) * TL::kTileBytes;
+    u32x4 kf[kKFrags];
+    static_for<0, kPF>([&](auto f) { kf[f] = lds_read_b128<(f % 2) * kKbOff + (f / 2) * kKsOff>(ka); });
+    static_for<0, kKFrags>([&](auto f) {
+      constexpr int kNewer = (kKFrags - 1 - f) < (kPF - 1) ? (kKFrags - 1 - f) : (kPF - 1);
+      wait_lgkm<kNewer>(kf[f]);
+      const Vec8 a = __builtin_bit_cast(Vec8, kf[f]);
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-      for (int qb = 0; qb < QB; ++qb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) s[kb][qb][r] = 0.f;
-    {
-      // K fragments stream through a short register queue: kPF reads ahead of the MFMA
-      // that consumes them, so LDS latency hides under the matrix pipeline.
-      constexpr int kFrags = 2 * KS;
-      constexpr int kPF = 4;
-      constexpr int kKbOff = (32 / RPB) * TL::kBlockPitch, kKsOff = 2 * TL::kChunkStride;
-      const uint32_t ka = static_cast<uint32_t>(k_rd + stage_idx * TL::kStageBytes);
-      u32x4 kf[kFrags];
-      static_for<0, kPF>([&](auto f) { kf[f] = lds_read_b128<(f / KS) * kKbOff + (f % KS) * kKsOff>(ka); });
-      static_for<0, kFrags>([&](auto f) {
-        constexpr int kNewer = (kFrags - 1 - f) < (kPF - 1) ? (kFrags - 1 - f) : (kPF - 1);
-        wait_lgkm<kNewer>(kf[f]);
-        const Vec8 a = __builtin_bit_cast(Vec8, kf[f]);
-#pragma unroll
-        for (int qb = 0; qb < QB; ++qb) s[f / KS][qb] = M::mma(a, qf[qb][f % KS], s[f / KS][qb]);
-        if constexpr (f + kPF < kFrags)
-          kf[f + kPF] = lds_read_b128<((f + kPF) / KS) * kKbOff + ((f + kPF) % KS) * kKsOff>(ka);
-      });
-    }
-
-    // V^T fragment queue (two transposing reads per fragment); the first kVPF fragments
-    // are requested now so that their latency hides under the softmax.
-    constexpr int kVFrags = 4 * DB;
-    constexpr int kVPF = 4;
-    const uint32_t va = static_cast<uint32_t>(v_rd + stage_idx * TL::kStageBytes + TL::kTileBytes);
+      for (int qb = 0; qb < QB; ++qb) {
+        if constexpr (f / 2 == 0) {
+          const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+          s[f % 2][qb] = M::mma(a, qf[qb][f / 2], zero);
+        } else {
+          s[f % 2][qb] = M::mma(a, qf[qb][f / 2], s[f % 2][qb]);
+        }
+      }
+      if constexpr (f + kPF < kKFrags) kf[f + kPF] = lds_read_b128<((f + kPF) % 2) * kKbOff + ((f + kPF) / 2) * kKsOff>(ka);
+    });
+  };
+  // O^T += V^T P^T of tile t.
+  auto pv_tile = [&](int t, const Vec8 (&pf)[QB][4]) __attribute__((always_inline)) {
+    const uint32_t va = v_rd + (t % NSV) * TL::kTileBytes;
     u32x2 vlo[kVFrags], vhi[kVFrags];
     auto issue_v = [&](auto g) __attribute__((always_inline)) {
       constexpr int kOff = (g / DB) * kVRowsOff16 + (g % DB) * 4 * TL::kChunkStride;
       vlo[g] = lds_read_tr16_b64<kOff>(va);
       vhi[g] = lds_read_tr16_b64<kOff + kVRowsOff8>(va);
     };
-    static_for<0, kVPF>(issue_v);
-
-    // online softmax; P^T packed to T in the B-operand layout of the P.V product
-    Vec8 pf[QB][4];
+    static_for<0, kPF>(issue_v);
+    static_for<0, kVFrags>([&](auto g) {
+      constexpr int kNewer = (kVFrags - 1 - g) < (kPF - 1) ? (kVFrags - 1 - g) : (kPF - 1);
+      wait_lgkm<2 * kNewer>(vlo[g], vhi[g]);
+      const s16x8 both = __builtin_shufflevector(__builtin_bit_cast(s16x4, vlo[g]), __builtin_bit_cast(s16x4, vhi[g]), 0, 1, 2, 3, 4, 5, 6, 7);
+      const Vec8 a = __builtin_bit_cast(Vec8, both);
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb) o[g % DB][qb] = M::mma(a, pf[qb][g / DB], o[g % DB][qb]);
+      if constexpr (g + kPF < kVFrags) issue_v(std::integral_constant<int, g + kPF>{});
+    });
+  };
+  // Both products of one pipelined iteration as ONE fragment stream: P.V of tile t-1
+  // (when HAS_PV) followed by K.Q of tile t+1, prefetching across the seam.
+  auto mma_stream = [&](auto has_pv_c, int t, const Vec8 (&pf)[QB][4], f32x16 (&s)[2][QB]) __attribute__((always_inline)) {
+    constexpr bool HAS_PV = decltype(has_pv_c)::value;
+    constexpr int NV = HAS_PV ? kVFrags : 0;
+    constexpr int NSTEP = NV + kKFrags;
+    const uint32_t va = v_rd + ((t + NSV - 1) % NSV) * TL::kTileBytes;   // tile t-1
+    const uint32_t ka = k_rd + ((t + 1) % NSK) * TL::kTileBytes;         // tile t+1
+    u32x2 vlo[kVFrags], vhi[kVFrags];
+    u32x4 kf[kKFrags];
+    auto issue = [&](auto i) __attribute__((always_inline)) {
+      if constexpr (i < NV) {
+        constexpr int g = i;
+        constexpr int kOff = (g / DB) * kVRowsOff16 + (g % DB) * 4 * TL::kChunkStride;
+        vlo[g] = lds_read_tr16_b64<kOff>(va);
+        vhi[g] = lds_read_tr16_b64<kOff + kVRowsOff8>(va);
+      } else {
+        constexpr int f = i - NV;
+        kf[f] = lds_read_b128<(f % 2) * kKbOff + (f / 2) * kKsOff>(ka);
+      }
+    };
+    static_for<0, kPF>(issue);
+    static_for<0, NSTEP>([&](auto i) {
+      // reads younger than step i's that are already queued: steps i+1 .. i+kPF-1
+      constexpr int kLast = (i + kPF - 1) < (NSTEP - 1) ? (i + kPF - 1) : (NSTEP - 1);
+      constexpr int kVNewer = (kLast < NV ? kLast : NV - 1) - (i < NV ? i : NV - 1);      // V steps in (i, kLast]
+      constexpr int kNewerReads = 2 * (kVNewer > 0 ? kVNewer : 0) + ((kLast - i) - (kVNewer > 0 ? kVNewer : 0));
+      if constexpr (i < NV) {
+        constexpr int g = i;
+        wait_lgkm<kNewerReads>(vlo[g], vhi[g]);
+        const s16x8 both = __builtin_shufflevector(__builtin_bit_cast(s16x4, vlo[g]), __builtin_bit_cast(s16x4, vhi[g]), 0, 1, 2, 3, 4, 5, 6, 7);
+        const Vec8 a = __builtin_bit_cast(Vec8, both);
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) o[g % DB][qb] = M::mma(a, pf[qb][g / DB], o[g % DB][qb]);
+      } else {
+        constexpr int f = i - NV;
+        wait_lgkm<kNewerReads>(kf[f]);
+        const Vec8 a = __builtin_bit_cast(Vec8, kf[f]);
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) {
+          if constexpr (f / 2 == 0) {
+            const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            s[f % 2][qb] = M::mma(a, qf[qb][f / 2], zero);
+          } else {
+            s[f % 2][qb] = M::mma(a, qf[qb][f / 2], s[f % 2][qb]);
+          }
+        }
+      }
+      if constexpr (i + kPF < NSTEP) issue(std::integral_constant<int, i + kPF>{});
+    });
+  };
+  // Online softmax of one tile's scores: updates m/l, leaves P^T packed to T in `pf` (the
+  // B-operand layout of the P.V product) and alpha in alpha_pending / rescale_pending
+  // (O is rescaled once the P.V product of the previous tile has been accumulated).
+  // MASKED tiles (tree block, ragged last cache tile) scale explicitly, add the mask,
+  // blank keys past the limit and keep the rounding residue of P in `s`.
+  auto softmax_tile = [&](auto masked_c, f32x16 (&s)[2][QB], Vec8 (&pf)[QB][4], bool tree, int key0, int key_lim) __attribute__((always_inline)) {
+    constexpr bool MASKED = decltype(masked_c)::value;
+    bool any_rescale = false;
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
       const float m_old = m_run[qb];
@@ -368,12 +427,8 @@ stage1_mfma_kernel(const KernelParams p) {
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int r = 0; r < 16; r += 2) {
-#ifdef FTA_DBG_NO_EXP
-          const float p0 = __builtin_fmaf(s[kb][qb][r], c, -m_use), p1 = __builtin_fmaf(s[kb][qb][r + 1], c, -m_use);
-#else
           const float p0 = MASKED ? fast_exp2(s[kb][qb][r] - m_use) : fast_exp2(__builtin_fmaf(s[kb][qb][r], c, -m_use));
           const float p1 = MASKED ? fast_exp2(s[kb][qb][r + 1] - m_use) : fast_exp2(__builtin_fmaf(s[kb][qb][r + 1], c, -m_use));
-#endif
           s[kb][qb][r] = p0;
           s[kb][qb][r + 1] = p1;
           ps0 += p0;
@@ -381,12 +436,8 @@ stage1_mfma_kernel(const KernelParams p) {
         }
       l_run[qb] = l_run[qb] * alpha + (ps0 + ps1);
       m_run[qb] = m_new;
-      if (__builtin_amdgcn_ballot_w64(m_new > m_old) != 0) {
-#pragma unroll
-        for (int db = 0; db < DB; ++db)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) o[db][qb][r] *= alpha;
-      }
+      alpha_pending[qb] = alpha;
+      any_rescale |= m_new > m_old;
 #pragma unroll
       for (int kk = 0; kk < 4; ++kk) {
         Vec8 pk;
@@ -404,85 +455,151 @@ stage1_mfma_kernel(const KernelParams p) {
         pf[qb][kk] = pk;
       }
     }
-
-    auto pv_product = [&]() __attribute__((always_inline)) {
-      static_for<0, kVFrags>([&](auto g) {
-        constexpr int kNewer = (kVFrags - 1 - g) < (kVPF - 1) ? (kVFrags - 1 - g) : (kVPF - 1);
-        wait_lgkm<2 * kNewer>(vlo[g], vhi[g]);
-        const s16x8 both = __builtin_shufflevector(__builtin_bit_cast(s16x4, vlo[g]), __builtin_bit_cast(s16x4, vhi[g]), 0, 1, 2, 3, 4, 5, 6, 7);
-        const Vec8 a = __builtin_bit_cast(Vec8, both);
+    rescale_pending = __builtin_amdgcn_ballot_w64(any_rescale) != 0;
+  };
+  auto apply_rescale = [&]() __attribute__((always_inline)) {
+    if (rescale_pending) {
 #pragma unroll
-        for (int qb = 0; qb < QB; ++qb) o[g % DB][qb] = M::mma(a, pf[qb][g / DB], o[g % DB][qb]);
-        if constexpr (g + kVPF < kVFrags) issue_v(std::integral_constant<int, g + kVPF>{});
-      });
-    };
-    pv_product();
-    if (MASKED) {
-      // Tree tiles and the ragged last cache tile are where single keys can carry large
-      // weights (short sequences); a second product with the low-order part of P removes
-      // the 2^-9 rounding of P there. Full cache tiles use one product.
+      for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) o[db][qb][r] *= alpha_pending[qb];
+      rescale_pending = false;
+    }
+  };
+  // Tile-boundary synchronisation at the top of iteration t: this wave's share of tile
+  // t+1 has landed, then the barrier (everybody's share has landed, and everybody is
+  // done with K(t) and V(t-2), whose stages tile t+NSK reuses), then tile t+NSK goes out.
+  auto tile_boundary = [&](int t) __attribute__((always_inline)) {
+    // loads younger than tile t+1's: tiles t+2 .. t+NSK-1 (those that exist)
+    const int younger = max(0, min(NSK - 2, ntiles - 2 - t));
+    if (NSK >= 4 && younger >= 2) wait_vmcnt<2 * kLoadsPerTile>();
+    else if (NSK >= 3 && younger >= 1) wait_vmcnt<kLoadsPerTile>();
+    else wait_vmcnt<0>();
+    __builtin_amdgcn_s_barrier();
+    if (t + NSK < ntiles) issue_tile(t + NSK);
+  };
+
+  // ---- the pipeline ----------------------------------------------------------------
+  // Iteration t runs the softmax of tile t on the vector ALU while the matrix pipeline
+  // works on P.V of tile t-1 and K.Q of tile t+1: two independent instruction streams in
+  // one basic block, interleaved by the scheduling hints below. Full cache tiles take
+  // this fused body; the ragged last cache tile and the tree tiles run the same three
+  // steps one after the other with the masked softmax.
+  // Buffers ping-pong between iterations (two statically unrolled roles) so that no
+  // register copies are needed: scores sA/sB, packed probabilities pA/pB.
+  f32x16 sA[2][QB], sB[2][QB];
+  Vec8 pA[QB][4], pB[QB][4];
+
+  // One fused iteration for full tile t: softmax(s_in) -> p_out on the vector ALU while
+  // the matrix pipeline does P.V of tile t-1 (p_in, when HAS_PV) and K.Q of tile t+1 -> s_out.
+  auto fused = [&](auto has_pv_c, int t, f32x16 (&s_in)[2][QB], f32x16 (&s_out)[2][QB], const Vec8 (&p_in)[QB][4], Vec8 (&p_out)[QB][4]) __attribute__((always_inline)) {
+    mma_stream(has_pv_c, t, p_in, s_out);
+    softmax_tile(std::false_type{}, s_in, p_out, false, kv_start + t * kKeyTile, kv_end);
+    // pace the two streams: a few vector-ALU instructions behind every MFMA
+#pragma unroll
+    for (int i = 0; i < (decltype(has_pv_c)::value ? kVFrags + kKFrags : kKFrags) * QB; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, decltype(has_pv_c)::value ? 6 : 12, 0);
+    }
+  };
+
+  // tile 0: wait for it (younger: tiles 1 .. NSK-1), barrier, scores -> sA.
+  {
+    const int younger = min(NSK - 1, ntiles - 1);
+    if (NSK >= 4 && younger >= 3) wait_vmcnt<3 * kLoadsPerTile>();
+    else if (NSK >= 3 && younger >= 2) wait_vmcnt<2 * kLoadsPerTile>();
+    else if (NSK >= 2 && younger >= 1) wait_vmcnt<kLoadsPerTile>();
+    else wait_vmcnt<0>();
+    __builtin_amdgcn_s_barrier();
+    if (wave_active) qk_tile(0, sA);
+  }
+
+  // fused iterations cover the full tiles that have a successor
+  const int fused_tiles = min(full_tiles, ntiles - 1);
+  int t = 0;
+  bool cur_in_B = false;   // which buffer pair holds the current scores / previous P
+  if (fused_tiles >= 1) {
+    tile_boundary(0);
+    if (wave_active) fused(std::false_type{}, 0, sA, sB, pB, pA);
+    t = 1;
+    cur_in_B = true;
+    for (; t + 1 < fused_tiles; t += 2) {
+      tile_boundary(t);
+      if (wave_active) {
+        apply_rescale();
+        fused(std::true_type{}, t, sB, sA, pA, pB);
+      }
+      tile_boundary(t + 1);
+      if (wave_active) {
+        apply_rescale();
+        fused(std::true_type{}, t + 1, sA, sB, pB, pA);
+      }
+    }
+    if (t < fused_tiles) {
+      tile_boundary(t);
+      if (wave_active) {
+        apply_rescale();
+        fused(std::true_type{}, t, sB, sA, pA, pB);
+      }
+      ++t;
+      cur_in_B = false;
+    }
+  }
+  // canonical roles for the tail: current scores in sB, previous P in pA
+  bool pv_pending = fused_tiles >= 1;   // P of tile t-1 has not been multiplied yet
+  bool prv_masked = false;
+  if (!cur_in_B) {
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb) sB[kb][qb] = sA[kb][qb];
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) pA[qb][kk] = pB[qb][kk];
+  }
+
+  // tail: the last tile of the split and every masked tile, step by step
+  auto pv_with_residue = [&](int tile, bool masked_prev) __attribute__((always_inline)) {
+    apply_rescale();
+    pv_tile(tile, pA);
+    if (masked_prev) {
+      // second, compensating product with the low-order part of P (parked in sA)
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) {
           Vec8 pk;
 #pragma unroll
-          for (int e = 0; e < 8; ++e) pk[e] = static_cast<T>(s[kk >> 1][qb][(kk & 1) * 8 + e]);
-          pf[qb][kk] = pk;
+          for (int e = 0; e < 8; ++e) pk[e] = static_cast<T>(sA[kk >> 1][qb][(kk & 1) * 8 + e]);
+          pA[qb][kk] = pk;
         }
-      static_for<0, kVPF>(issue_v);
-      pv_product();
+      pv_tile(tile, pA);
     }
   };
-
-  // ---- the pipeline: tiles t+1 .. t+NS-1 are in flight (HBM -> LDS) while tile t is
-  // consumed. Per tile: wait until this wave's share of tile t has landed, barrier
-  // (everybody's share has landed AND everybody is done with tile t-1, whose stage is
-  // the one the next load reuses), issue tile t+NS-1, compute tile t.
-#pragma unroll
-  for (int t = 0; t < NS - 1; ++t)
-    if (t < ntiles) issue_tile(t);
-
-  auto wait_tile = [&](int t) __attribute__((always_inline)) {
-    // loads issued after tile t's: min(NS-2, ntiles-1-t) tiles of kLoadsPerTile each
-    const int ahead = min(NS - 2, ntiles - 1 - t);
-    if (NS >= 4 && ahead >= 2) wait_vmcnt<2 * kLoadsPerTile>();
-    else if (NS >= 3 && ahead >= 1) wait_vmcnt<kLoadsPerTile>();
-    else wait_vmcnt<0>();
-  };
-
-  FTA_STAMP();
-  int t = 0;
-  for (; t < full_tiles; ++t) {
-#ifdef FTA_DBG_NO_GLOBAL
-    wait_vmcnt<0>();
-#ifndef FTA_DBG_NO_BARRIER
-    __builtin_amdgcn_s_barrier();
-#endif
-#else
-    wait_tile(t);
-#ifndef FTA_DBG_NO_BARRIER
-    __builtin_amdgcn_s_barrier();
-#endif
-    if (t + NS - 1 < ntiles) issue_tile(t + NS - 1);
-#endif
-#ifndef FTA_DBG_NO_COMPUTE
-    if (wave_active) process_tile(std::false_type{}, t % NS, false, kv_start + t * kKeyTile, kv_end);
-#endif
-  }
-  FTA_STAMP();
   for (; t < ntiles; ++t) {
-    wait_tile(t);
-    FTA_STAMP();
-    __builtin_amdgcn_s_barrier();
-    if (t + NS - 1 < ntiles) issue_tile(t + NS - 1);
+    tile_boundary(t);
+    if (!wave_active) continue;
+    const bool masked = t >= full_tiles;
     const bool tree = t >= cache_tiles;
     const int key0 = tree ? (t - cache_tiles) * kKeyTile : kv_start + t * kKeyTile;
-    if (wave_active) process_tile(std::true_type{}, t % NS, tree, key0, tree ? L : kv_end);
+    if (pv_pending) pv_with_residue(t - 1, prv_masked);
+    if (masked) softmax_tile(std::true_type{}, sB, pA, tree, key0, tree ? L : kv_end);
+    else softmax_tile(std::false_type{}, sB, pA, false, key0, kv_end);
+    // a masked tile leaves the rounding residue of P in sB: park it in sA, the scores of
+    // tile t+1 go to sB
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb) sA[kb][qb] = sB[kb][qb];
+    if (t + 1 < ntiles) qk_tile(t + 1, sB);
+    pv_pending = true;
+    prv_masked = masked;
   }
-
-  FTA_STAMP();
   if (!wave_active) return;
+  if (pv_pending) pv_with_residue(ntiles - 1, prv_masked);
 
   // ---- epilogue
   const bool direct = p.num_splits == 1;
@@ -520,19 +637,11 @@ stage1_mfma_kernel(const KernelParams p) {
       }
     }
   }
-#ifdef FTA_DBG_TIMING
-  FTA_STAMP();
-  if (tid == 0 && (blockIdx.x == 0 || blockIdx.x == 255)) {
-    long long* dst = reinterpret_cast<long long*>(p.mid_lse) + (blockIdx.x == 0 ? 0 : 16);
-    for (int i = 0; i < dbg_n; ++i) dst[i] = dbg_t[i];
-    dst[15] = dbg_n; dst[14] = clock64() - dbg_c0;
-  }
-#endif
 }
 
 template <typename T, int D, int QB, int NW, int NS>
 int launch(const KernelParams& p, hipStream_t stream) {
-  constexpr int kSmem = NS * TileLayout<D>::kStageBytes;
+  constexpr int kSmem = (2 * NS + 2) * TileLayout<D>::kTileBytes;  // K ring of NS stages + V ring of NS + 2
   static_assert(kSmem <= 160 * 1024, "LDS budget");
   auto kern = stage1_mfma_kernel<T, D, QB, NW, NS>;
   if (kSmem > 64 * 1024) {
@@ -554,12 +663,12 @@ int launch(const KernelParams& p, hipStream_t stream) {
 
 template <typename T>
 int launch_t(const KernelParams& p, int head_dim, hipStream_t stream) {
-  if (p.rows_per_wg == 256) {  // 8 waves, one workgroup per CU, 4-stage ring
-    if (head_dim == 128) return launch<T, 128, 1, 8, 4>(p, stream);
-    if (head_dim == 64) return launch<T, 64, 1, 8, 4>(p, stream);
-  } else if (p.rows_per_wg == 128) {  // 4 waves, two workgroups per CU, 2-stage ring each
-    if (head_dim == 128) return launch<T, 128, 1, 4, 2>(p, stream);
-    if (head_dim == 64) return launch<T, 64, 1, 4, 2>(p, stream);
+  if (p.rows_per_wg == 256) {  // 8 waves, one workgroup per CU, K ring 3 / V ring 5
+    if (head_dim == 128) return launch<T, 128, 1, 8, 3>(p, stream);
+    if (head_dim == 64) return launch<T, 64, 1, 8, 3>(p, stream);
+  } else if (p.rows_per_wg == 128) {  // 4 waves, same rings
+    if (head_dim == 128) return launch<T, 128, 1, 4, 3>(p, stream);
+    if (head_dim == 64) return launch<T, 64, 1, 4, 3>(p, stream);
   }
   return FTA_ERR_UNSUPPORTED;
 }
