@@ -10,13 +10,14 @@
 
 namespace fta {
 
-// One MFMA workgroup holds 128 query rows (4 waves x 32). Two such workgroups share a
-// CU; they synchronise independently, so one's softmax overlaps the other's MFMAs.
-// FTA_ROWS_PER_WG=256 selects the 8-wave, 256-row variant (tuning only).
+// Query rows one MFMA workgroup holds: 256 (8 waves x 32 rows, two waves per SIMD)
+// when the unit has more than 128 rows, else 128 (4 waves). One workgroup per CU either
+// way (the K/V rings take most of the LDS). FTA_ROWS_PER_WG=128 forces the 4-wave
+// variant (tuning only).
 int mfma_rows_per_wg(int rows) {
   if (const char* env = std::getenv("FTA_ROWS_PER_WG"))
-    if (std::atoi(env) == 256 && rows > 128) return 256;
-  return 128;
+    if (std::atoi(env) == 128) return 128;
+  return rows > 128 ? 256 : 128;
 }
 
 namespace {
@@ -216,6 +217,8 @@ int decode_impl(const fta_args* args, void* hip_stream, int stages) {
   p.cur_group = a.num_q_heads / a.cur_heads;
   p.rows = pl.rows_per_group; p.rows_per_wg = pl.rows_per_wg; p.row_blocks = pl.row_blocks;
   p.len_is_i64 = a.len_dtype == FTA_I64;
+  p.mask_vec4 = reinterpret_cast<uintptr_t>(a.mask) % 16 == 0 && a.mask_stride[0] % 4 == 0 && a.mask_stride[1] % 4 == 0 &&
+                a.mask_stride[2] % 4 == 0;
   p.scale_log2 = a.sm_scale * fta::kLog2e;
   for (int i = 0; i < 3; ++i) {
     p.q_stride[i] = a.q_stride[i]; p.k_stride[i] = a.k_stride[i]; p.v_stride[i] = a.v_stride[i];

@@ -39,6 +39,7 @@ struct KernelParams {
   int32_t rows_per_wg;
   int32_t row_blocks;
   int32_t len_is_i64;
+  int32_t mask_vec4;      // every mask row starts 16-byte aligned
   float scale_log2;       // sm_scale * log2(e)
 
   int64_t q_stride[3];

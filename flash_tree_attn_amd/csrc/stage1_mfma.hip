@@ -28,6 +28,7 @@
 // (current_k / current_v with the additive mask), which replaces the eager block and
 // sigmoid merge of flash_tree_attn.py:367-373. Output: the final result (one split)
 // or a normalised fp32 partial plus its log-sum-exp (flash_tree_attn.py:121-144).
+#include <cstdlib>
 #include <type_traits>
 
 #include "fta_device.h"
@@ -149,6 +150,13 @@ stage1_mfma_kernel(const KernelParams p) {
   constexpr int kVRing = NSK * TL::kTileBytes;       // byte offset of the V ring
 
   extern __shared__ __attribute__((aligned(16))) char smem[];
+#ifdef FTA_DBG_TIMING
+  long long dbg_t[12]; int dbg_n = 0; const long long dbg_c0 = clock64();
+#define FTA_STAMP() do { if (dbg_n < 12) dbg_t[dbg_n++] = wall_clock64(); } while (0)
+#else
+#define FTA_STAMP() do {} while (0)
+#endif
+  FTA_STAMP();
 
   const WorkItem w = decode_work(p, blockIdx.x);
   const int b = w.batch;
@@ -178,10 +186,13 @@ stage1_mfma_kernel(const KernelParams p) {
   const char* ckbase = reinterpret_cast<const char*>(static_cast<const T*>(p.ck) + b * p.ck_stride[0] + cur_head * p.ck_stride[1]);
   const char* cvbase = reinterpret_cast<const char*>(static_cast<const T*>(p.cv) + b * p.cv_stride[0] + cur_head * p.cv_stride[1]);
 
+  // Tile order: the tree tiles first (their masked, latency-bound handling overlaps the
+  // ramp-up of the cache stream), then the cache tiles of this split; only the last cache
+  // tile can be ragged.
   const int cache_tiles = kv_end > kv_start ? (kv_end - kv_start + kKeyTile - 1) / kKeyTile : 0;
   const int full_tiles = kv_end > kv_start ? (kv_end - kv_start) / kKeyTile : 0;
   const int tree_tiles = owns_tree ? (L + kKeyTile - 1) / kKeyTile : 0;
-  const int ntiles = cache_tiles + tree_tiles;
+  const int ntiles = tree_tiles + cache_tiles;
 
   // ---- Q fragments (B operand of S^T = K Q^T), kept in registers for the whole split
   Vec8 qf[QB][KS];
@@ -215,7 +226,7 @@ stage1_mfma_kernel(const KernelParams p) {
   auto issue_full_tile = [&](int t) __attribute__((always_inline)) {
     char* kst = smem + (t % NSK) * TL::kTileBytes;
     char* vst = smem + kVRing + (t % NSV) * TL::kTileBytes;
-    const int key0 = kv_start + t * kKeyTile;
+    const int key0 = kv_start + (t - tree_tiles) * kKeyTile;
 #pragma unroll
     for (int i = 0; i < kLoadsPerTensor; ++i) {
       const int blk = i * NW + wave;
@@ -230,8 +241,8 @@ stage1_mfma_kernel(const KernelParams p) {
   auto issue_edge_tile = [&](int t) __attribute__((always_inline)) {
     char* kst = smem + (t % NSK) * TL::kTileBytes;
     char* vst = smem + kVRing + (t % NSV) * TL::kTileBytes;
-    const bool tree = t >= cache_tiles;
-    const int key0 = tree ? (t - cache_tiles) * kKeyTile : kv_start + t * kKeyTile;
+    const bool tree = t < tree_tiles;
+    const int key0 = tree ? t * kKeyTile : kv_start + (t - tree_tiles) * kKeyTile;
     const int key_lim = tree ? L : kv_end;
     const char* kb_ = tree ? ckbase : kbase;
     const char* vb_ = tree ? cvbase : vbase;
@@ -245,17 +256,39 @@ stage1_mfma_kernel(const KernelParams p) {
       __builtin_amdgcn_global_load_lds((const FTA_GLOBAL void*)(vb_ + j * vrb + ld_chunk * 16), (FTA_LDS void*)(vst + blk * TL::kBlockPitch), 16, 0, 0);
     }
   };
-  auto issue_tile = [&](int t) __attribute__((always_inline)) {
-    if (t < full_tiles) issue_full_tile(t); else issue_edge_tile(t);
+  // Tiles are requested in order. A tile may go out once the stage it lands in is free:
+  // tile j reuses the K stage of tile j-NSK and the V stage of tile j-NSV. `k_done` /
+  // `v_done` count the tiles whose K / V every wave has finished reading (as of the last
+  // barrier).
+  int next_issue = 0;
+  auto issue_ready = [&](int k_done, int v_done) __attribute__((always_inline)) {
+    while (next_issue < ntiles && next_issue - k_done < NSK && next_issue - v_done < NSV) {
+      const int t = next_issue++;
+      if (t >= tree_tiles && t - tree_tiles < full_tiles) issue_full_tile(t); else issue_edge_tile(t);
+    }
+  };
+  // One synchronisation point: this wave's share of tile `need` has landed (tiles land in
+  // request order; `need` < 0 waits for nothing), then the barrier (everybody's share has
+  // landed, and everybody is past the reads that k_done / v_done describe), then every
+  // tile whose stages have become free is requested.
+  auto sync_point = [&](int need, int k_done, int v_done) __attribute__((always_inline)) {
+    if (need >= 0) {
+      const int younger = next_issue - 1 - need;   // tiles requested after `need`
+      if (younger >= 4) wait_vmcnt<4 * kLoadsPerTile>();
+      else if (younger == 3) wait_vmcnt<3 * kLoadsPerTile>();
+      else if (younger == 2) wait_vmcnt<2 * kLoadsPerTile>();
+      else if (younger == 1) wait_vmcnt<kLoadsPerTile>();
+      else wait_vmcnt<0>();
+    }
+    __builtin_amdgcn_s_barrier();
+    issue_ready(k_done, v_done);
   };
 
   // Q must have landed before the tile loop: a pending register load inside the loop
   // would make the compiler drain ALL vector-memory traffic (vmcnt 0) every iteration,
-  // including the K/V tiles that are meant to stay in flight. Then the first NSK tiles go out.
+  // including the K/V tiles that are meant to stay in flight. Then the first tiles go out.
   wait_vmcnt<0>();
-#pragma unroll
-  for (int t = 0; t < NSK; ++t)
-    if (t < ntiles) issue_tile(t);
+  issue_ready(0, 0);
 
   f32x16 o[DB][QB];
   float m_run[QB], l_run[QB], alpha_pending[QB];
@@ -328,7 +361,7 @@ stage1_mfma_kernel(const KernelParams p) {
   };
   // Both products of one pipelined iteration as ONE fragment stream: P.V of tile t-1
   // (when HAS_PV) followed by K.Q of tile t+1, prefetching across the seam.
-  auto mma_stream = [&](auto has_pv_c, int t, const Vec8 (&pf)[QB][4], f32x16 (&s)[2][QB]) __attribute__((always_inline)) {
+  auto mma_stream = [&](auto has_pv_c, int t, const Vec8 (&pf)[QB][4], f32x16 (&s)[2][QB], auto&& valu_slice) __attribute__((always_inline)) {
     constexpr bool HAS_PV = decltype(has_pv_c)::value;
     constexpr int NV = HAS_PV ? kVFrags : 0;
     constexpr int NSTEP = NV + kKFrags;
@@ -375,40 +408,55 @@ stage1_mfma_kernel(const KernelParams p) {
         }
       }
       if constexpr (i + kPF < NSTEP) issue(std::integral_constant<int, i + kPF>{});
+      // the vector-ALU work that runs in this MFMA's shadow; the fence keeps the compiler
+      // from regrouping the two streams (it would put all MFMAs first)
+      valu_slice(i, std::integral_constant<int, NSTEP>{});
+      __builtin_amdgcn_sched_barrier(0);
     });
+  };
+  // Additive mask values of one tree tile in the accumulator layout (lane = query row,
+  // 16 registers = 4 groups of 4 consecutive keys per 32-key block). Indices are clamped
+  // instead of branched on, so all loads of a tile are in flight together; rows that
+  // start 16-byte aligned fetch each group of 4 keys with one 128-bit load.
+  auto load_mask = [&](int key0, float (&mv)[QB][2][16]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+      const float* mrow = p.mask + b * p.mask_stride[0] + row_head[qb] * p.mask_stride[1] + row_i[qb] * p.mask_stride[2];
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {
+          const int j0 = key0 + kb * 32 + rg * 8 + 4 * lh;
+          if (p.mask_vec4 && j0 + 3 < L) {
+            const f32x4 v4 = *reinterpret_cast<const f32x4*>(mrow + j0);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) mv[qb][kb][rg * 4 + e] = v4[e];
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) mv[qb][kb][rg * 4 + e] = mrow[min(j0 + e, L - 1)];
+          }
+        }
+    }
   };
   // Online softmax of one tile's scores: updates m/l, leaves P^T packed to T in `pf` (the
   // B-operand layout of the P.V product) and alpha in alpha_pending / rescale_pending
   // (O is rescaled once the P.V product of the previous tile has been accumulated).
   // MASKED tiles (tree block, ragged last cache tile) scale explicitly, add the mask,
   // blank keys past the limit and keep the rounding residue of P in `s`.
-  auto softmax_tile = [&](auto masked_c, f32x16 (&s)[2][QB], Vec8 (&pf)[QB][4], bool tree, int key0, int key_lim) __attribute__((always_inline)) {
+  auto softmax_tile = [&](auto masked_c, f32x16 (&s)[2][QB], Vec8 (&pf)[QB][4], bool tree, int key0, int key_lim, const float (&mv)[QB][2][16]) __attribute__((always_inline)) {
     constexpr bool MASKED = decltype(masked_c)::value;
     bool any_rescale = false;
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
       const float m_old = m_run[qb];
       if (MASKED) {
-        // Mask values are fetched with clamped indices and no branches, so that all of a
-        // tile's loads are in flight together (one memory round trip, not one per value).
-        float mv[2][16];
-        if (tree) {
-          const float* mrow = p.mask + b * p.mask_stride[0] + row_head[qb] * p.mask_stride[1] + row_i[qb] * p.mask_stride[2];
-#pragma unroll
-          for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const int j = key0 + kb * 32 + (r >> 2) * 8 + 4 * lh + (r & 3);
-              mv[kb][r] = mrow[min(j, key_lim - 1)];
-            }
-        }
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             const int j = key0 + kb * 32 + (r >> 2) * 8 + 4 * lh + (r & 3);
             float sv = s[kb][qb][r] * c;
-            if (tree) sv = __builtin_fmaf(mv[kb][r], kLog2e, sv);
+            if (tree) sv = __builtin_fmaf(mv[qb][kb][r], kLog2e, sv);
             s[kb][qb][r] = j < key_lim ? sv : neg_inf();
           }
       }
@@ -468,19 +516,6 @@ stage1_mfma_kernel(const KernelParams p) {
       rescale_pending = false;
     }
   };
-  // Tile-boundary synchronisation at the top of iteration t: this wave's share of tile
-  // t+1 has landed, then the barrier (everybody's share has landed, and everybody is
-  // done with K(t) and V(t-2), whose stages tile t+NSK reuses), then tile t+NSK goes out.
-  auto tile_boundary = [&](int t) __attribute__((always_inline)) {
-    // loads younger than tile t+1's: tiles t+2 .. t+NSK-1 (those that exist)
-    const int younger = max(0, min(NSK - 2, ntiles - 2 - t));
-    if (NSK >= 4 && younger >= 2) wait_vmcnt<2 * kLoadsPerTile>();
-    else if (NSK >= 3 && younger >= 1) wait_vmcnt<kLoadsPerTile>();
-    else wait_vmcnt<0>();
-    __builtin_amdgcn_s_barrier();
-    if (t + NSK < ntiles) issue_tile(t + NSK);
-  };
-
   // ---- the pipeline ----------------------------------------------------------------
   // Iteration t runs the softmax of tile t on the vector ALU while the matrix pipeline
   // works on P.V of tile t-1 and K.Q of tile t+1: two independent instruction streams in
@@ -495,50 +530,119 @@ stage1_mfma_kernel(const KernelParams p) {
   // One fused iteration for full tile t: softmax(s_in) -> p_out on the vector ALU while
   // the matrix pipeline does P.V of tile t-1 (p_in, when HAS_PV) and K.Q of tile t+1 -> s_out.
   auto fused = [&](auto has_pv_c, int t, f32x16 (&s_in)[2][QB], f32x16 (&s_out)[2][QB], const Vec8 (&p_in)[QB][4], Vec8 (&p_out)[QB][4]) __attribute__((always_inline)) {
-    mma_stream(has_pv_c, t, p_in, s_out);
-    softmax_tile(std::false_type{}, s_in, p_out, false, kv_start + t * kKeyTile, kv_end);
-    // pace the two streams: a few vector-ALU instructions behind every MFMA
+    // The lean softmax (full tile: no mask, no key limit) cut into slices, one per MFMA
+    // step: steps [0, NA) take the row maximum, step NA exchanges it between the half
+    // waves and fixes the new maximum, the following steps exponentiate and pack pairs
+    // of values, the last step updates the running sum.
+    float mx0[QB], mx1[QB], m_new[QB], alpha[QB], ps0[QB], ps1[QB];
+    auto slice = [&](auto i_c, auto nstep_c) __attribute__((always_inline)) {
+      constexpr int I = decltype(i_c)::value, NSTEP = decltype(nstep_c)::value;
+      constexpr int NA = NSTEP / 4, EPA = 32 / NA;
+      constexpr int NC = NSTEP - NA - 1, PPS = (16 + NC - 1) / NC;
 #pragma unroll
-    for (int i = 0; i < (decltype(has_pv_c)::value ? kVFrags + kKFrags : kKFrags) * QB; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, decltype(has_pv_c)::value ? 6 : 12, 0);
+      for (int qb = 0; qb < QB; ++qb) {
+        if constexpr (I < NA) {
+#pragma unroll
+          for (int x = I * EPA; x < (I + 1) * EPA; x += 2) {
+            const float a0 = s_in[x / 16][qb][x % 16], a1 = s_in[x / 16][qb][x % 16 + 1];
+            mx0[qb] = (x == 0) ? a0 : fmaxf(mx0[qb], a0);
+            mx1[qb] = (x == 0) ? a1 : fmaxf(mx1[qb], a1);
+          }
+        } else if constexpr (I == NA) {
+          const float mx = half_swap_max(fmaxf(mx0[qb], mx1[qb]), lh);
+          m_new[qb] = fmaxf(m_run[qb], mx * c);
+          alpha[qb] = fast_exp2(m_run[qb] - m_new[qb]);
+          ps0[qb] = 0.f;
+          ps1[qb] = 0.f;
+        } else {
+          constexpr int J0 = (I - NA - 1) * PPS;
+#pragma unroll
+          for (int j = J0; j < J0 + PPS && j < 16; ++j) {
+            const int x = 2 * j, kb = x / 16, r = x % 16;
+            const float p0 = fast_exp2(__builtin_fmaf(s_in[kb][qb][r], c, -m_new[qb]));
+            const float p1 = fast_exp2(__builtin_fmaf(s_in[kb][qb][r + 1], c, -m_new[qb]));
+            ps0[qb] += p0;
+            ps1[qb] += p1;
+            const f32x2 pv = {p0, p1};
+            const auto pr = __builtin_convertvector(pv, typename M::Vec2);
+            p_out[qb][kb * 2 + (r >= 8)][r % 8] = pr[0];
+            p_out[qb][kb * 2 + (r >= 8)][r % 8 + 1] = pr[1];
+          }
+        }
+      }
+      if constexpr (I == NSTEP - 1) {
+        bool any_rescale = false;
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) {
+          l_run[qb] = l_run[qb] * alpha[qb] + (ps0[qb] + ps1[qb]);
+          any_rescale |= m_new[qb] > m_run[qb];
+          m_run[qb] = m_new[qb];
+          alpha_pending[qb] = alpha[qb];
+        }
+        rescale_pending = __builtin_amdgcn_ballot_w64(any_rescale) != 0;
+      }
+    };
+    mma_stream(has_pv_c, t, p_in, s_out, slice);
+  };
+
+  // second, compensating P.V product of a masked tile: P's rounding residue is in `res`
+  auto pv_with_residue = [&](int tile, bool masked_tile, f32x16 (&res)[2][QB]) __attribute__((always_inline)) {
+    apply_rescale();
+    pv_tile(tile, pA);
+    if (masked_tile) {
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+          Vec8 pk;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) pk[e] = static_cast<T>(res[kk >> 1][qb][(kk & 1) * 8 + e]);
+          pA[qb][kk] = pk;
+        }
+      pv_tile(tile, pA);
     }
   };
 
-  // tile 0: wait for it (younger: tiles 1 .. NSK-1), barrier, scores -> sA.
-  {
-    const int younger = min(NSK - 1, ntiles - 1);
-    if (NSK >= 4 && younger >= 3) wait_vmcnt<3 * kLoadsPerTile>();
-    else if (NSK >= 3 && younger >= 2) wait_vmcnt<2 * kLoadsPerTile>();
-    else if (NSK >= 2 && younger >= 1) wait_vmcnt<kLoadsPerTile>();
-    else wait_vmcnt<0>();
-    __builtin_amdgcn_s_barrier();
-    if (wave_active) qk_tile(0, sA);
+  float mask_vals[QB][2][16];
+  // phase A: the tree tiles, one complete step each (scores, masked softmax, P.V twice)
+  const int c0 = tree_tiles;   // first cache tile
+  for (int u = 0; u < tree_tiles; ++u) {
+    sync_point(u, u, u);
+    if (!wave_active) continue;
+    load_mask(u * kKeyTile, mask_vals);   // in flight while the scores are computed
+    qk_tile(u, sB);
+    softmax_tile(std::true_type{}, sB, pA, true, u * kKeyTile, L, mask_vals);
+    pv_with_residue(u, true, sB);
   }
+  FTA_STAMP();
 
-  // fused iterations cover the full tiles that have a successor
-  const int fused_tiles = min(full_tiles, ntiles - 1);
-  int t = 0;
+  // phase B: fused iterations over the full cache tiles that have a successor
+  const int fused_cnt = cache_tiles >= 1 ? min(full_tiles, cache_tiles - 1) : 0;
+  int t = c0;
   bool cur_in_B = false;   // which buffer pair holds the current scores / previous P
-  if (fused_tiles >= 1) {
-    tile_boundary(0);
-    if (wave_active) fused(std::false_type{}, 0, sA, sB, pB, pA);
-    t = 1;
+  if (cache_tiles >= 1) {
+    sync_point(c0, c0, c0);
+    if (wave_active) qk_tile(c0, sA);
+  }
+  if (fused_cnt >= 1) {
+    sync_point(c0 + 1, c0 + 1, c0);
+    if (wave_active) fused(std::false_type{}, c0, sA, sB, pB, pA);
+    t = c0 + 1;
     cur_in_B = true;
-    for (; t + 1 < fused_tiles; t += 2) {
-      tile_boundary(t);
+    for (; t + 1 < c0 + fused_cnt; t += 2) {
+      sync_point(t + 1, t + 1, max(c0, t - 1));
       if (wave_active) {
         apply_rescale();
         fused(std::true_type{}, t, sB, sA, pA, pB);
       }
-      tile_boundary(t + 1);
+      sync_point(t + 2, t + 2, max(c0, t));
       if (wave_active) {
         apply_rescale();
         fused(std::true_type{}, t + 1, sA, sB, pB, pA);
       }
     }
-    if (t < fused_tiles) {
-      tile_boundary(t);
+    if (t < c0 + fused_cnt) {
+      sync_point(t + 1, t + 1, max(c0, t - 1));
       if (wave_active) {
         apply_rescale();
         fused(std::true_type{}, t, sB, sA, pA, pB);
@@ -547,8 +651,9 @@ stage1_mfma_kernel(const KernelParams p) {
       cur_in_B = false;
     }
   }
+  FTA_STAMP();
   // canonical roles for the tail: current scores in sB, previous P in pA
-  bool pv_pending = fused_tiles >= 1;   // P of tile t-1 has not been multiplied yet
+  bool pv_pending = fused_cnt >= 1;   // P of tile t-1 has not been multiplied yet
   bool prv_masked = false;
   if (!cur_in_B) {
 #pragma unroll
@@ -561,33 +666,14 @@ stage1_mfma_kernel(const KernelParams p) {
       for (int kk = 0; kk < 4; ++kk) pA[qb][kk] = pB[qb][kk];
   }
 
-  // tail: the last tile of the split and every masked tile, step by step
-  auto pv_with_residue = [&](int tile, bool masked_prev) __attribute__((always_inline)) {
-    apply_rescale();
-    pv_tile(tile, pA);
-    if (masked_prev) {
-      // second, compensating product with the low-order part of P (parked in sA)
-#pragma unroll
-      for (int qb = 0; qb < QB; ++qb)
-#pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-          Vec8 pk;
-#pragma unroll
-          for (int e = 0; e < 8; ++e) pk[e] = static_cast<T>(sA[kk >> 1][qb][(kk & 1) * 8 + e]);
-          pA[qb][kk] = pk;
-        }
-      pv_tile(tile, pA);
-    }
-  };
+  // phase C: the last cache tiles of the split, step by step (the last one may be ragged)
   for (; t < ntiles; ++t) {
-    tile_boundary(t);
+    sync_point(t + 1 < ntiles ? t + 1 : -1, t + 1, max(c0, t - 1));
     if (!wave_active) continue;
-    const bool masked = t >= full_tiles;
-    const bool tree = t >= cache_tiles;
-    const int key0 = tree ? (t - cache_tiles) * kKeyTile : kv_start + t * kKeyTile;
-    if (pv_pending) pv_with_residue(t - 1, prv_masked);
-    if (masked) softmax_tile(std::true_type{}, sB, pA, tree, key0, tree ? L : kv_end);
-    else softmax_tile(std::false_type{}, sB, pA, false, key0, kv_end);
+    const bool masked = t - c0 >= full_tiles;
+    if (pv_pending) pv_with_residue(t - 1, prv_masked, sA);
+    if (masked) softmax_tile(std::true_type{}, sB, pA, false, kv_start + (t - c0) * kKeyTile, kv_end, mask_vals);
+    else softmax_tile(std::false_type{}, sB, pA, false, kv_start + (t - c0) * kKeyTile, kv_end, mask_vals);
     // a masked tile leaves the rounding residue of P in sB: park it in sA, the scores of
     // tile t+1 go to sB
 #pragma unroll
@@ -599,7 +685,8 @@ stage1_mfma_kernel(const KernelParams p) {
     prv_masked = masked;
   }
   if (!wave_active) return;
-  if (pv_pending) pv_with_residue(ntiles - 1, prv_masked);
+  if (pv_pending) pv_with_residue(ntiles - 1, prv_masked, sA);
+  FTA_STAMP();
 
   // ---- epilogue
   const bool direct = p.num_splits == 1;
@@ -637,6 +724,14 @@ stage1_mfma_kernel(const KernelParams p) {
       }
     }
   }
+#ifdef FTA_DBG_TIMING
+  FTA_STAMP();
+  if (tid == 0 && (blockIdx.x == 0 || blockIdx.x == gridDim.x - 1)) {
+    long long* dst = reinterpret_cast<long long*>(p.mid_lse) + (blockIdx.x == 0 ? 0 : 16);
+    for (int i = 0; i < dbg_n; ++i) dst[i] = dbg_t[i];
+    dst[15] = dbg_n; dst[14] = clock64() - dbg_c0;
+  }
+#endif
 }
 
 template <typename T, int D, int QB, int NW, int NS>
@@ -664,6 +759,8 @@ int launch(const KernelParams& p, hipStream_t stream) {
 template <typename T>
 int launch_t(const KernelParams& p, int head_dim, hipStream_t stream) {
   if (p.rows_per_wg == 256) {  // 8 waves, one workgroup per CU, K ring 3 / V ring 5
+    if (const char* env = std::getenv("FTA_QB2"))  // tuning: 4 waves x 64 rows, one wave per SIMD
+      if (std::atoi(env) == 1 && head_dim == 128) return launch<T, 128, 2, 4, 3>(p, stream);
     if (head_dim == 128) return launch<T, 128, 1, 8, 3>(p, stream);
     if (head_dim == 64) return launch<T, 64, 1, 8, 3>(p, stream);
   } else if (p.rows_per_wg == 128) {  // 4 waves, same rings
