@@ -31,6 +31,8 @@ def parse():
     ap.add_argument("--kv-sets", type=int, default=0, help="independent KV caches to rotate over (0 = enough for >1 GiB)")
     ap.add_argument("--splits", type=int, default=0, help="pin the split count (0 = heuristic)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run plain device copies of a known size (reference point for rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
     return ap.parse_args()
 
@@ -99,6 +101,16 @@ def main():
     cfg = CONFIGS[args.config]
     dev = "cuda:0"
     torch.cuda.set_device(0)
+    if args.copy_calibration:
+        nbytes_copy = 1 << 30
+        src = torch.empty(nbytes_copy // 2, dtype=torch.bfloat16, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(max(args.steps, 1)):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration": True, "bytes_read_per_copy": nbytes_copy, "bytes_written_per_copy": nbytes_copy,
+                          "copies": max(args.steps, 1)}))
+        return
     esz = torch.empty((), dtype=cfg.dtype).element_size()
     kv_bytes = 2 * cfg.bsz * cfg.num_kv_heads * cfg.cache_len * cfg.head_dim * esz
     kv_sets = args.kv_sets or max(2, min(8, -(-(1 << 30) // kv_bytes)))

@@ -759,8 +759,6 @@ int launch(const KernelParams& p, hipStream_t stream) {
 template <typename T>
 int launch_t(const KernelParams& p, int head_dim, hipStream_t stream) {
   if (p.rows_per_wg == 256) {  // 8 waves, one workgroup per CU, K ring 3 / V ring 5
-    if (const char* env = std::getenv("FTA_QB2"))  // tuning: 4 waves x 64 rows, one wave per SIMD
-      if (std::atoi(env) == 1 && head_dim == 128) return launch<T, 128, 2, 4, 3>(p, stream);
     if (head_dim == 128) return launch<T, 128, 1, 8, 3>(p, stream);
     if (head_dim == 64) return launch<T, 64, 1, 8, 3>(p, stream);
   } else if (p.rows_per_wg == 128) {  // 4 waves, same rings
