@@ -40,10 +40,10 @@ __device__ __forceinline__ int splits_for(int t, int chunk, int num_splits) {
 }
 
 struct WorkItem {
-  int split, unit, batch, row_block;
+  int item, unit, row_block;  // item = (sequence, split) pair, see item_by_order
 };
 
-// Linear workgroup id -> (split, row_block, unit, batch).
+// Linear workgroup id -> (unit, row_block, item).
 // Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2. The row
 // blocks of one (batch, unit, split) read the same K/V stream, so they are given ids
 // that differ by a multiple of 8 and land on the same XCD: the second block's K/V
@@ -66,10 +66,66 @@ __device__ __forceinline__ WorkItem decode_work(const KernelParams& p, int id) {
   }
   WorkItem w;
   w.row_block = rb;
-  w.split = g % p.num_splits; g /= p.num_splits;
+  // Units vary fastest: the XCDs are served strictly round-robin, so the 8 workgroups of
+  // one dispatch round must carry equal work, and the units of one (sequence, split) do.
+  // A split index that varied with the XCD would starve the XCDs of the high splits on
+  // ragged batches, where short sequences fill only the first splits.
   w.unit = g % p.units;
-  w.batch = g / p.units;
+  w.item = g / p.units;
   return w;
+}
+
+// Longest-first dispatch for ragged batches. Workgroup ids are handed out in order, and
+// round-robin at every level of the machine (XCD, then shader engine), so any run of
+// consecutive ids should carry near-equal work and the heaviest items should come first.
+// Item k (from the workgroup id) is therefore resolved against the batch's lengths:
+// first every full chunk (all equal work; sequence-major), then the last chunk of every
+// sequence (partial chunk + tree block) in descending size; what remains of the grid has
+// nothing to do. No host look at the lengths and no atomics: every workgroup recomputes
+// the order from the bsz lengths in one LDS pass. Batches of one sequence or beyond
+// kMaxOrderedBatch keep the identity order. Returns false if the item is empty. Must be
+// called by all threads of the block.
+constexpr int kMaxOrderedBatch = 256;
+__device__ __forceinline__ bool item_by_order(const KernelParams& p, int k, int* batch, int* split) {
+  if (p.bsz == 1 || p.bsz > kMaxOrderedBatch) {
+    *batch = k / p.num_splits;
+    *split = k % p.num_splits;
+    return true;
+  }
+  __shared__ int s_nsp[kMaxOrderedBatch];
+  __shared__ int s_tail[kMaxOrderedBatch];
+  __shared__ int s_pick[2];
+  const int t = threadIdx.x;
+  for (int i = t; i < p.bsz; i += blockDim.x) {
+    const int64_t v = load_len(p.lens, p.len_is_i64, i);
+    const int len = static_cast<int>(v < 0 ? 0 : (v > p.cache_len ? p.cache_len : v));
+    const int n = splits_for(len, p.chunk, p.num_splits);
+    s_nsp[i] = n;
+    s_tail[i] = len - (n - 1) * p.chunk;
+  }
+  if (t == 0) s_pick[0] = -1;
+  __syncthreads();
+  for (int i = t; i < p.bsz; i += blockDim.x) {
+    const int mine = s_tail[i];
+    int before = 0, total = 0, rank = 0;
+    for (int j = 0; j < p.bsz; ++j) {
+      const int f = s_nsp[j] - 1;
+      total += f;
+      before += j < i ? f : 0;
+      rank += (s_tail[j] > mine) || (s_tail[j] == mine && j < i);
+    }
+    if (k >= before && k < before + s_nsp[i] - 1) {
+      s_pick[0] = i;
+      s_pick[1] = k - before;
+    } else if (k - total == rank) {
+      s_pick[0] = i;
+      s_pick[1] = s_nsp[i] - 1;
+    }
+  }
+  __syncthreads();
+  *batch = __builtin_amdgcn_readfirstlane(s_pick[0]);  // uniform: keep them in scalar registers
+  *split = __builtin_amdgcn_readfirstlane(s_pick[1]);
+  return *batch >= 0;
 }
 
 __device__ __forceinline__ float wave_max(float x) {

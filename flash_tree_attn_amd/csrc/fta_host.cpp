@@ -3,6 +3,7 @@
 // machine without a GPU can exercise them.
 #include <hip/hip_runtime_api.h>
 
+#include <cmath>
 #include <algorithm>
 #include <cstdlib>
 
@@ -90,23 +91,36 @@ int plan(const fta_args& a, int num_cus, fta_plan_out* out) {
   const int64_t t_cap = a.max_seq_len_hint > 0 ? std::min(a.max_seq_len_hint, a.cache_len) : a.cache_len;
   const int gran = std::max(a.block_size, kKeyTile);
 
-  // A split costs one fp32 partial written by stage 1 and read back by stage 2; in
-  // units of "keys of K/V traffic" that is 2*rows*D*4 / (2*D*esize) keys.
-  const int64_t partial_keys = 4LL * std::min(rows, rows_per_wg) / esize(a.dtype);
-  const int64_t min_chunk_fill = std::max<int64_t>(gran, 4 * kKeyTile);          // when CUs would idle otherwise
-  const int64_t min_chunk_over = std::max<int64_t>(min_chunk_fill, 8 * partial_keys);  // when only balancing
-
+  // Split count from a cost model of one launch, in microseconds, with every sequence
+  // taken at the length cap (lengths are not known on the host):
+  //   rounds(S) * wg(S) + tail * wg(S) + merge(S),   wg(S) = fixed + tile_us * tiles(S)
+  // rounds = workgroups / CUs rounded up (one workgroup per CU), `fixed` the measured
+  // per-workgroup prologue + tree step + epilogue, `tile_us` the steady-state time of
+  // one 64-key tile with every CU busy, `tail` the expected idle share of the last
+  // round of a ragged batch (a single sequence has nothing to balance), merge the
+  // fp32 partials written and read back. Few long chunks win over many short ones:
+  // the fixed part is worth 7-10 tiles.
   const int64_t target = static_cast<int64_t>(num_cus) * wg_per_cu;
-  int64_t s_fill = cdiv(target, work_items);
-  s_fill = std::min(s_fill, std::max<int64_t>(1, t_cap / min_chunk_fill));
-  // Ragged batches: lengths are not known on the host, so oversubscribe the CUs
-  // with equal-sized chunks; a single sequence has nothing to balance.
-  int64_t s_over = 1;
-  if (a.bsz > 1) {
-    s_over = cdiv(8 * target, work_items);
-    s_over = std::min(s_over, std::max<int64_t>(1, t_cap / min_chunk_over));
+  const int64_t min_chunk = std::max<int64_t>(gran, 4 * kKeyTile);
+  const int64_t s_max = std::max<int64_t>(1, std::min<int64_t>(64, std::max<int64_t>(t_cap, 1) / min_chunk));
+  const double fixed_us = 20.0;
+  const double tile_us = kernel == FTA_KERNEL_MFMA ? (rows_per_wg > 128 ? 2.85 : 2.2) : 0.6 * rows_per_wg;
+  const double tree_tiles = 3.0 * cdiv(a.q_len, kKeyTile);
+  const double tail_share = a.bsz > 1 ? 0.25 : 0.0;
+  const double partial_mb = 4e-6 * a.bsz * a.num_q_heads * a.q_len * a.head_dim;  // MB per split slot
+  int64_t splits = 1;
+  double best = 0.0;
+  for (int64_t cand = 1; cand <= s_max; ++cand) {
+    const double tiles = std::ceil((std::max<int64_t>(t_cap, 1) / static_cast<double>(kKeyTile) + tree_tiles) / cand);
+    const double wg_us = fixed_us + tile_us * tiles;
+    const double rounds = static_cast<double>(cdiv(work_items * cand, target));
+    const double merge_us = cand > 1 ? 6.0 + cand * partial_mb / 4.0 : 0.0;
+    const double cost = (rounds + tail_share) * wg_us + merge_us;
+    if (cand == 1 || cost < best * 0.98) {  // a larger count has to win by 2 %
+      best = cost;
+      splits = cand;
+    }
   }
-  int64_t splits = std::max<int64_t>(1, std::max(s_fill, s_over));
   if (a.force_splits > 0) splits = a.force_splits;
   if (const char* env = std::getenv("FTA_FORCE_SPLITS")) {
     const int v = std::atoi(env);
@@ -115,7 +129,15 @@ int plan(const fta_args& a, int num_cus, fta_plan_out* out) {
   // Never more splits than blocks of the reference granularity, so that a scratch
   // buffer sized like the reference's (flash_tree_attn.py:274-281) always fits.
   splits = std::min<int64_t>(splits, std::max<int64_t>(1, cdiv(t_cap, gran)));
-  int64_t chunk = cdiv(cdiv(std::max<int64_t>(t_cap, 1), splits), gran) * gran;
+  // The split that owns the end of a sequence also processes the tree block (a masked,
+  // latency-bound step worth about three cache tiles per tree tile): count it as extra
+  // keys when cutting chunks, so that the last split of a full-length sequence gets a
+  // correspondingly shorter cache range.
+  int64_t tree_weight = 3;
+  if (const char* env = std::getenv("FTA_TREE_TILE_WEIGHT")) tree_weight = std::max(0, std::atoi(env));
+  const int64_t tree_keys = splits > 1 ? tree_weight * kKeyTile * cdiv(a.q_len, kKeyTile) : 0;
+  int64_t chunk = cdiv(cdiv(std::max<int64_t>(t_cap, 1) + tree_keys, splits), gran) * gran;
+  if ((splits - 1) * chunk >= std::max<int64_t>(t_cap, 1)) chunk = cdiv(cdiv(std::max<int64_t>(t_cap, 1), splits), gran) * gran;
   splits = std::max<int64_t>(1, cdiv(std::max<int64_t>(t_cap, 1), chunk));
 
   out->kernel = kernel;

@@ -159,14 +159,15 @@ stage1_mfma_kernel(const KernelParams p) {
   FTA_STAMP();
 
   const WorkItem w = decode_work(p, blockIdx.x);
-  const int b = w.batch;
+  int b, split;
+  if (!item_by_order(p, w.item, &b, &split)) return;
   int64_t t64 = load_len(p.lens, p.len_is_i64, b);
   const int T_b = static_cast<int>(t64 < 0 ? 0 : (t64 > p.cache_len ? p.cache_len : t64));
   const int S_b = splits_for(T_b, p.chunk, p.num_splits);
-  if (w.split >= S_b) return;
-  const int kv_start = w.split * p.chunk;
-  const int kv_end = (w.split == p.num_splits - 1) ? T_b : min(T_b, kv_start + p.chunk);
-  const bool owns_tree = (w.split == S_b - 1);
+  if (split >= S_b) return;
+  const int kv_start = split * p.chunk;
+  const int kv_end = (split == p.num_splits - 1) ? T_b : min(T_b, kv_start + p.chunk);
+  const bool owns_tree = (split == S_b - 1);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -264,6 +265,9 @@ stage1_mfma_kernel(const KernelParams p) {
   auto issue_ready = [&](int k_done, int v_done) __attribute__((always_inline)) {
     while (next_issue < ntiles && next_issue - k_done < NSK && next_issue - v_done < NSV) {
       const int t = next_issue++;
+#ifdef FTA_DBG_NO_DMA
+      if (t >= NSK) continue;
+#endif
       if (t >= tree_tiles && t - tree_tiles < full_tiles) issue_full_tile(t); else issue_edge_tile(t);
     }
   };
@@ -315,7 +319,10 @@ stage1_mfma_kernel(const KernelParams p) {
   constexpr int kKbOff = (32 / RPB) * TL::kBlockPitch, kKsOff = 2 * TL::kChunkStride;
   constexpr int kKFrags = 2 * KS;   // K fragments per tile (one 128-bit read each)
   constexpr int kVFrags = 4 * DB;   // V^T fragments per tile (two transposing reads each)
-  constexpr int kPF = 4;            // fragments requested ahead of the MFMA that consumes them
+#ifndef FTA_PF
+#define FTA_PF 4
+#endif
+  constexpr int kPF = FTA_PF;       // fragments requested ahead of the MFMA that consumes them
 
   // ---- building blocks -------------------------------------------------------------
   // S^T = K Q^T of tile t (fragment queue: kPF reads ahead of the consuming MFMA).
@@ -373,11 +380,15 @@ stage1_mfma_kernel(const KernelParams p) {
       if constexpr (i < NV) {
         constexpr int g = i;
         constexpr int kOff = (g / DB) * kVRowsOff16 + (g % DB) * 4 * TL::kChunkStride;
+#ifndef FTA_DBG_NO_VREAD
         vlo[g] = lds_read_tr16_b64<kOff>(va);
         vhi[g] = lds_read_tr16_b64<kOff + kVRowsOff8>(va);
+#endif
       } else {
         constexpr int f = i - NV;
+#ifndef FTA_DBG_NO_KREAD
         kf[f] = lds_read_b128<(f % 2) * kKbOff + (f / 2) * kKsOff>(ka);
+#endif
       }
     };
     static_for<0, kPF>(issue);
@@ -392,26 +403,42 @@ stage1_mfma_kernel(const KernelParams p) {
         const s16x8 both = __builtin_shufflevector(__builtin_bit_cast(s16x4, vlo[g]), __builtin_bit_cast(s16x4, vhi[g]), 0, 1, 2, 3, 4, 5, 6, 7);
         const Vec8 a = __builtin_bit_cast(Vec8, both);
 #pragma unroll
+#ifndef FTA_DBG_NO_MMA
         for (int qb = 0; qb < QB; ++qb) o[g % DB][qb] = M::mma(a, pf[qb][g / DB], o[g % DB][qb]);
+#else
+        for (int qb = 0; qb < QB; ++qb) o[g % DB][qb][0] += (float)a[0];
+#endif
       } else {
         constexpr int f = i - NV;
         wait_lgkm<kNewerReads>(kf[f]);
         const Vec8 a = __builtin_bit_cast(Vec8, kf[f]);
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb) {
+#ifndef FTA_DBG_NO_MMA
           if constexpr (f / 2 == 0) {
             const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
             s[f % 2][qb] = M::mma(a, qf[qb][f / 2], zero);
           } else {
             s[f % 2][qb] = M::mma(a, qf[qb][f / 2], s[f % 2][qb]);
           }
+#else
+          s[f % 2][qb][f / 2] = (float)a[0];
+#endif
         }
       }
+#ifndef FTA_DBG_NO_LDSREAD
       if constexpr (i + kPF < NSTEP) issue(std::integral_constant<int, i + kPF>{});
+#else
+      if constexpr (i + kPF < NSTEP && i < kPF) issue(std::integral_constant<int, i + kPF>{});
+#endif
       // the vector-ALU work that runs in this MFMA's shadow; the fence keeps the compiler
       // from regrouping the two streams (it would put all MFMAs first)
+#ifndef FTA_DBG_NO_SLICE
       valu_slice(i, std::integral_constant<int, NSTEP>{});
+#endif
+#ifndef FTA_DBG_NO_FENCE
       __builtin_amdgcn_sched_barrier(0);
+#endif
     });
   };
   // Additive mask values of one tree tile in the accumulator layout (lane = query row,
@@ -708,7 +735,7 @@ stage1_mfma_kernel(const KernelParams p) {
           *reinterpret_cast<typename M::Vec4*>(dst + db * 32 + rg * 8 + 4 * lh) = v4;
         }
     } else {
-      float* dst = p.mid_o + b * p.mid_o_stride[0] + head * p.mid_o_stride[1] + w.split * p.mid_o_stride[2] + i * p.mid_o_stride[3];
+      float* dst = p.mid_o + b * p.mid_o_stride[0] + head * p.mid_o_stride[1] + split * p.mid_o_stride[2] + i * p.mid_o_stride[3];
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -720,7 +747,7 @@ stage1_mfma_kernel(const KernelParams p) {
         }
       if (lh == 0) {
         const float lse = l_tot > 0.f ? (m_run[qb] + fast_log2(l_tot)) * kLn2 : neg_inf();
-        p.mid_lse[b * p.mid_lse_stride[0] + head * p.mid_lse_stride[1] + w.split * p.mid_lse_stride[2] + i] = lse;
+        p.mid_lse[b * p.mid_lse_stride[0] + head * p.mid_lse_stride[1] + split * p.mid_lse_stride[2] + i] = lse;
       }
     }
   }

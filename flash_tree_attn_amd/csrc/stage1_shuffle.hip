@@ -41,14 +41,15 @@ __global__ void __launch_bounds__(256) stage1_shuffle_kernel(const KernelParams 
   float* Ps = reinterpret_cast<float*>(smem + S::kKBytes + S::kVBytes + S::kQBytes);
 
   const WorkItem w = decode_work(p, blockIdx.x);
-  const int b = w.batch;
+  int b, split;
+  if (!item_by_order(p, w.item, &b, &split)) return;
   int64_t t64 = load_len(p.lens, p.len_is_i64, b);
   const int T_b = static_cast<int>(t64 < 0 ? 0 : (t64 > p.cache_len ? p.cache_len : t64));
   const int S_b = splits_for(T_b, p.chunk, p.num_splits);
-  if (w.split >= S_b) return;
-  const int kv_start = w.split * p.chunk;
-  const int kv_end = (w.split == p.num_splits - 1) ? T_b : min(T_b, kv_start + p.chunk);
-  const bool owns_tree = (w.split == S_b - 1);
+  if (split >= S_b) return;
+  const int kv_start = split * p.chunk;
+  const int kv_end = (split == p.num_splits - 1) ? T_b : min(T_b, kv_start + p.chunk);
+  const bool owns_tree = (split == S_b - 1);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -189,13 +190,13 @@ __global__ void __launch_bounds__(256) stage1_shuffle_kernel(const KernelParams 
       if (direct) {
         static_cast<T*>(p.out)[b * p.out_stride[0] + head * p.out_stride[1] + i * p.out_stride[2] + d] = static_cast<T>(o);
       } else {
-        p.mid_o[b * p.mid_o_stride[0] + head * p.mid_o_stride[1] + w.split * p.mid_o_stride[2] +
+        p.mid_o[b * p.mid_o_stride[0] + head * p.mid_o_stride[1] + split * p.mid_o_stride[2] +
                 i * p.mid_o_stride[3] + d] = o;
       }
     }
     if (!direct && lane == 0) {
       const float lse = l_run[rr] > 0.f ? (m_run[rr] + fast_log2(l_run[rr])) * kLn2 : neg_inf();
-      p.mid_lse[b * p.mid_lse_stride[0] + head * p.mid_lse_stride[1] + w.split * p.mid_lse_stride[2] + i] = lse;
+      p.mid_lse[b * p.mid_lse_stride[0] + head * p.mid_lse_stride[1] + split * p.mid_lse_stride[2] + i] = lse;
     }
   }
 }

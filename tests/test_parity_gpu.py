@@ -281,6 +281,26 @@ def test_lengths_beyond_cache_are_clamped_and_padding_is_ignored():
     check(run(x), ref, torch.bfloat16)
 
 
+@pytest.mark.parametrize("bsz,splits", [(37, 1), (37, 3), (37, 4), (64, 8), (300, 2)])
+def test_ragged_batch_dispatch_order(bsz, splits):
+    """Stage 1 resolves its workgroups longest-first from the batch's lengths; every
+    (sequence, split) must still be computed exactly once whatever the order: ties, empty
+    caches, lengths that are exact multiples of the chunk, and batches beyond the limit
+    of the ordered dispatch (identity order)."""
+    g = torch.Generator().manual_seed(bsz * 31 + splits)
+    tmax = 512
+    lens = torch.randint(0, tmax + 1, (bsz,), generator=g).tolist()
+    lens[0], lens[1], lens[2], lens[3] = 0, tmax, tmax, 0
+    chunk = -(-tmax // splits // 64) * 64
+    for i, mult in enumerate(range(1, splits + 1)):
+        if 4 + i < bsz and mult * chunk <= tmax:
+            lens[4 + i] = mult * chunk
+    x = make(51, bsz, 4, 2, 8, 64, tmax, torch.float16, lens)
+    ref = oracle(x)
+    check(run(x, _force_splits=splits), ref, torch.float16)
+    check(run(x, _force_splits=splits, _force_kernel=_lib.KERNEL_SHUFFLE), ref, torch.float16)
+
+
 # ---------------------------------------------------------------- size-independent properties
 def test_properties_at_headline_size():
     cfg = CONFIGS["cfg3_gqa_8b_bf16"]
