@@ -7,7 +7,7 @@ import os
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libfta.so")
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 FTA_F32, FTA_F16, FTA_BF16 = 0, 1, 2
 FTA_I32, FTA_I64 = 0, 1
 KERNEL_SHUFFLE, KERNEL_MFMA = 0, 1
@@ -26,11 +26,12 @@ class FtaArgs(C.Structure):
         ("q", C.c_void_p), ("k_cache", C.c_void_p), ("v_cache", C.c_void_p),
         ("cur_k", C.c_void_p), ("cur_v", C.c_void_p), ("mask", C.c_void_p),
         ("kv_seq_len", C.c_void_p), ("out", C.c_void_p), ("mid_o", C.c_void_p), ("mid_lse", C.c_void_p),
+        ("counters", C.c_void_p),
         ("bsz", C.c_int32), ("num_q_heads", C.c_int32), ("num_kv_heads", C.c_int32), ("cur_heads", C.c_int32),
         ("q_len", C.c_int32), ("head_dim", C.c_int32), ("cache_len", C.c_int32), ("v_cache_len", C.c_int32),
         ("block_size", C.c_int32), ("max_seq_len_hint", C.c_int32), ("mid_splits", C.c_int32),
         ("dtype", C.c_int32), ("len_dtype", C.c_int32), ("force_splits", C.c_int32), ("force_kernel", C.c_int32),
-        ("sm_scale", C.c_float),
+        ("counter_elems", C.c_int32), ("sm_scale", C.c_float),
         ("q_stride", C.c_int64 * 3), ("k_stride", C.c_int64 * 3), ("v_stride", C.c_int64 * 3),
         ("ck_stride", C.c_int64 * 3), ("cv_stride", C.c_int64 * 3), ("mask_stride", C.c_int64 * 3),
         ("out_stride", C.c_int64 * 3), ("mid_o_stride", C.c_int64 * 4), ("mid_lse_stride", C.c_int64 * 3),
@@ -40,7 +41,8 @@ class FtaArgs(C.Structure):
 class FtaPlanOut(C.Structure):
     _fields_ = [
         ("kernel", C.c_int32), ("num_splits", C.c_int32), ("chunk", C.c_int32), ("rows_per_group", C.c_int32),
-        ("rows_per_wg", C.c_int32), ("row_blocks", C.c_int32), ("num_workgroups", C.c_int32), ("reserved", C.c_int32),
+        ("rows_per_wg", C.c_int32), ("row_blocks", C.c_int32), ("num_workgroups", C.c_int32), ("counter_elems", C.c_int32),
+        ("single_launch", C.c_int32), ("reserved", C.c_int32),
         ("mid_o_elems", C.c_int64), ("mid_lse_elems", C.c_int64),
     ]
 

@@ -148,6 +148,11 @@ int plan(const fta_args& a, int num_cus, fta_plan_out* out) {
   out->row_blocks = row_blocks;
   out->num_workgroups = static_cast<int32_t>(work_items * splits);
   out->reserved = 0;
+  out->counter_elems = (splits > 1 && kernel == FTA_KERNEL_MFMA && work_items <= 0x7fffffff) ? static_cast<int32_t>(work_items) : 0;
+  // Merging inside stage 1 saves the second launch, but the last workgroup of a sequence
+  // merges alone: that pays with two splits and one round of workgroups (short launches,
+  // where the second kernel and the gap before it weigh most), not beyond.
+  out->single_launch = out->counter_elems > 0 && splits <= 2 && work_items * splits <= target;
   out->mid_lse_elems = splits > 1 ? static_cast<int64_t>(a.bsz) * a.num_q_heads * splits * a.q_len : 0;
   out->mid_o_elems = out->mid_lse_elems * a.head_dim;
   return FTA_OK;
@@ -227,10 +232,14 @@ int decode_impl(const fta_args* args, void* hip_stream, int stages) {
       if (a.mid_lse_stride[i] < 0) return FTA_ERR_STRIDE;
     if (reinterpret_cast<uintptr_t>(a.mid_o) % 16 != 0) return FTA_ERR_STRIDE;
   }
+  // Single launch: only for the whole path, and only where the plan has such a path.
+  const bool fused = stages == 3 && a.counters != nullptr && pl.counter_elems > 0;
+  if (fused && a.counter_elems < pl.counter_elems) return FTA_ERR_SCRATCH_TOO_SMALL;
 
   fta::KernelParams p{};
   p.q = a.q; p.k = a.k_cache; p.v = a.v_cache; p.ck = a.cur_k; p.cv = a.cur_v;
   p.mask = a.mask; p.lens = a.kv_seq_len; p.out = a.out; p.mid_o = a.mid_o; p.mid_lse = a.mid_lse;
+  p.counters = fused ? a.counters : nullptr;
   p.bsz = a.bsz; p.num_q_heads = a.num_q_heads; p.q_len = a.q_len; p.cache_len = a.cache_len;
   p.chunk = pl.chunk; p.num_splits = pl.num_splits;
   p.heads_per_unit = pl.rows_per_group / a.q_len;
@@ -254,7 +263,7 @@ int decode_impl(const fta_args* args, void* hip_stream, int stages) {
     st = pl.kernel == FTA_KERNEL_MFMA ? fta::launch_stage1_mfma(p, a.dtype, a.head_dim, hip_stream)
                                       : fta::launch_stage1_shuffle(p, a.dtype, a.head_dim, hip_stream);
   if (st) return st;
-  if ((stages & 2) && pl.num_splits > 1) st = fta::launch_stage2_merge(p, a.dtype, a.head_dim, hip_stream);
+  if ((stages & 2) && pl.num_splits > 1 && !fused) st = fta::launch_stage2_merge(p, a.dtype, a.head_dim, hip_stream);
   return st;
 }
 }  // namespace

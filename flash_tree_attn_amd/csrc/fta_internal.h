@@ -24,6 +24,7 @@ struct KernelParams {
   void* out;
   float* mid_o;
   float* mid_lse;
+  int32_t* counters;      // one per (sequence, unit, row block) when the merge runs inside stage 1, else null
 
   int32_t bsz;
   int32_t num_q_heads;

@@ -111,6 +111,29 @@ __device__ __forceinline__ u32x2 lds_read_tr16_b64(uint32_t addr) {
   asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
   return v;
 }
+// Register load the compiler's wait insertion does not see (same reason as above: a
+// load it tracks forces vmcnt 0 once tile requests of unknown number follow it). The
+// caller waits with wait_vmcnt and then passes the registers through settle().
+template <int OFF>
+__device__ __forceinline__ u32x4 global_read_b128(const void* ptr) {
+  u32x4 v;
+  asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=&v"(v) : "v"(ptr), "n"(OFF) : "memory");
+  return v;
+}
+__device__ __forceinline__ void settle(u32x4& a) { asm volatile("" : "+v"(a)); }
+// Device-scope (sc1) 128-bit store / load: the store writes through to the point where
+// every XCD sees it, the load is never served from a stale line of this XCD's caches.
+// They carry the partials that one workgroup hands to another inside a launch without
+// any cache-wide writeback or invalidate. Untracked like the reads above: wait_vmcnt.
+__device__ __forceinline__ void store_b128_device(void* ptr, f32x4 v) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(ptr), "v"(v) : "memory");
+}
+__device__ __forceinline__ f32x4 load_b128_device(const void* ptr) {
+  f32x4 v;
+  asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=&v"(v) : "v"(ptr) : "memory");
+  return v;
+}
+__device__ __forceinline__ void settle(f32x4& a) { asm volatile("" : "+v"(a)); }
 template <int N>
 __device__ __forceinline__ void wait_lgkm(u32x4& a) {
   asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(a) : "n"(N));
@@ -197,21 +220,17 @@ stage1_mfma_kernel(const KernelParams p) {
 
   // ---- Q fragments (B operand of S^T = K Q^T), kept in registers for the whole split
   Vec8 qf[QB][KS];
+  u32x4 qraw[QB][KS];
   bool row_ok[QB];
   int row_head[QB], row_i[QB];
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
     const int row = wave_row0 + qb * 32 + li;
     row_ok[qb] = row < p.rows;
-    row_head[qb] = head0 + (row_ok[qb] ? row / L : 0);
+    row_head[qb] = head0 + (row_ok[qb] ? row / L : 0);   // rows past the end read row 0 and are zeroed below
     row_i[qb] = row_ok[qb] ? row % L : 0;
-    const T* qrow = static_cast<const T*>(p.q) + b * p.q_stride[0] + row_head[qb] * p.q_stride[1] + row_i[qb] * p.q_stride[2];
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      u32x4 raw = {0, 0, 0, 0};
-      if (row_ok[qb]) raw = *reinterpret_cast<const u32x4*>(qrow + 16 * ks + 8 * lh);
-      qf[qb][ks] = __builtin_bit_cast(Vec8, raw);
-    }
+    const T* qrow = static_cast<const T*>(p.q) + b * p.q_stride[0] + row_head[qb] * p.q_stride[1] + row_i[qb] * p.q_stride[2] + 8 * lh;
+    static_for<0, KS>([&](auto ks) { qraw[qb][ks] = global_read_b128<32 * ks>(qrow); });
   }
 
   // ---- HBM -> LDS: lane i of a wave-wide load fetches chunk i/RPB of row i%RPB of one
@@ -288,11 +307,21 @@ stage1_mfma_kernel(const KernelParams p) {
     issue_ready(k_done, v_done);
   };
 
-  // Q must have landed before the tile loop: a pending register load inside the loop
-  // would make the compiler drain ALL vector-memory traffic (vmcnt 0) every iteration,
-  // including the K/V tiles that are meant to stay in flight. Then the first tiles go out.
-  wait_vmcnt<0>();
+  // The first tiles go out right behind the Q loads, so that both latencies overlap;
+  // then wait for Q alone: everything younger is this wave's share of those tiles.
   issue_ready(0, 0);
+  if (next_issue >= 3) wait_vmcnt<3 * kLoadsPerTile>();
+  else if (next_issue == 2) wait_vmcnt<2 * kLoadsPerTile>();
+  else if (next_issue == 1) wait_vmcnt<kLoadsPerTile>();
+  else wait_vmcnt<0>();
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      settle(qraw[qb][ks]);
+      const u32x4 zero = {0, 0, 0, 0};
+      qf[qb][ks] = __builtin_bit_cast(Vec8, row_ok[qb] ? qraw[qb][ks] : zero);
+    }
 
   f32x16 o[DB][QB];
   float m_run[QB], l_run[QB], alpha_pending[QB];
@@ -716,12 +745,23 @@ stage1_mfma_kernel(const KernelParams p) {
   FTA_STAMP();
 
   // ---- epilogue
-  const bool direct = p.num_splits == 1;
+  // One split (of the launch, or of this sequence when the merge runs in this kernel):
+  // the normalised result goes straight to `out`. Otherwise the normalised partial and
+  // its log-sum-exp go to the scratch buffers, to be merged by stage 2 or, with
+  // counters, by whichever workgroup of the sequence finishes last (below).
+  const bool merge_here = p.counters != nullptr;
+  const bool direct = p.num_splits == 1 || (merge_here && S_b == 1);
+  float lse_own[QB];
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
     const float l_tot = half_swap_sum(l_run[qb], lh);
-    if (!row_ok[qb]) continue;
+    lse_own[qb] = l_tot > 0.f ? (m_run[qb] + fast_log2(l_tot)) * kLn2 : neg_inf();
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[db][qb][r] *= inv;
+    if (!row_ok[qb]) continue;
     const int head = row_head[qb], i = row_i[qb];
     if (direct) {
       T* dst = static_cast<T*>(p.out) + b * p.out_stride[0] + head * p.out_stride[1] + i * p.out_stride[2];
@@ -731,7 +771,7 @@ stage1_mfma_kernel(const KernelParams p) {
         for (int rg = 0; rg < 4; ++rg) {
           typename M::Vec4 v4;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) v4[e] = static_cast<T>(o[db][qb][rg * 4 + e] * inv);
+          for (int e = 0; e < 4; ++e) v4[e] = static_cast<T>(o[db][qb][rg * 4 + e]);
           *reinterpret_cast<typename M::Vec4*>(dst + db * 32 + rg * 8 + 4 * lh) = v4;
         }
     } else {
@@ -742,13 +782,96 @@ stage1_mfma_kernel(const KernelParams p) {
         for (int rg = 0; rg < 4; ++rg) {
           f32x4 v4;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) v4[e] = o[db][qb][rg * 4 + e] * inv;
-          *reinterpret_cast<f32x4*>(dst + db * 32 + rg * 8 + 4 * lh) = v4;
+          for (int e = 0; e < 4; ++e) v4[e] = o[db][qb][rg * 4 + e];
+          if (merge_here) store_b128_device(dst + db * 32 + rg * 8 + 4 * lh, v4);
+          else *reinterpret_cast<f32x4*>(dst + db * 32 + rg * 8 + 4 * lh) = v4;
         }
       if (lh == 0) {
-        const float lse = l_tot > 0.f ? (m_run[qb] + fast_log2(l_tot)) * kLn2 : neg_inf();
-        p.mid_lse[b * p.mid_lse_stride[0] + head * p.mid_lse_stride[1] + split * p.mid_lse_stride[2] + i] = lse;
+        float* lse_dst = p.mid_lse + b * p.mid_lse_stride[0] + head * p.mid_lse_stride[1] + split * p.mid_lse_stride[2] + i;
+        if (merge_here) __hip_atomic_store(lse_dst, lse_own[qb], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else *lse_dst = lse_own[qb];
       }
+    }
+  }
+
+  // ---- merge inside this launch (flash_tree_attn.py:339-365 without a second kernel).
+  // Every workgroup of a (sequence, unit, row block) bumps that group's counter once its
+  // partial has been written through (device-scope stores, all acknowledged); the one
+  // that sees S_b - 1 is the last, resets the counter for the next call and merges: its
+  // own partial from registers, the others from scratch with device-scope loads. No
+  // workgroup ever waits for another, and no cache is flushed or invalidated as a whole.
+  if (merge_here && !direct) {
+    __shared__ int s_last;
+    wait_vmcnt<0>();      // this thread's partial stores are acknowledged ...
+    __syncthreads();      // ... and so are those of every thread of the workgroup
+    if (tid == 0) {
+      int32_t* cnt = p.counters + (static_cast<int64_t>(b) * p.units + w.unit) * p.row_blocks + w.row_block;
+      const int old = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const int last = old == S_b - 1;
+      if (last) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      s_last = last;
+    }
+    __syncthreads();
+    if (!s_last) return;
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+      if (!row_ok[qb]) continue;
+      const int head = row_head[qb], i = row_i[qb];
+      const float* lse_p = p.mid_lse + b * p.mid_lse_stride[0] + head * p.mid_lse_stride[1] + i;
+      const float* mo = p.mid_o + b * p.mid_o_stride[0] + head * p.mid_o_stride[1] + i * p.mid_o_stride[3] + 4 * lh;
+      // log-sum-exp of the other splits: the first four in one round trip, kept for the weights
+      float lse_c[4];
+#pragma unroll
+      for (int s = 0; s < 4; ++s)
+        lse_c[s] = (s < S_b && s != split) ? __hip_atomic_load(lse_p + s * p.mid_lse_stride[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                                           : neg_inf();
+      float mx = fmaxf(fmaxf(lse_own[qb], fmaxf(lse_c[0], lse_c[1])), fmaxf(lse_c[2], lse_c[3]));
+      for (int s = 4; s < S_b; ++s)
+        if (s != split) mx = fmaxf(mx, __hip_atomic_load(lse_p + s * p.mid_lse_stride[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+      float wsum = 0.f;
+      if (mx != neg_inf()) {
+        const float w_own = fast_exp2((lse_own[qb] - mx) * kLog2e);
+        wsum = w_own;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) o[db][qb][r] *= w_own;
+        for (int s = 0; s < S_b; ++s) {
+          if (s == split) continue;
+          const float lse_s = s == 0 ? lse_c[0] : s == 1 ? lse_c[1] : s == 2 ? lse_c[2] : s == 3 ? lse_c[3]
+                            : __hip_atomic_load(lse_p + s * p.mid_lse_stride[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          const float wgt = fast_exp2((lse_s - mx) * kLog2e);
+          wsum += wgt;
+          const float* src = mo + s * p.mid_o_stride[2];
+          f32x4 part[DB][4];
+#pragma unroll
+          for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int rg = 0; rg < 4; ++rg) part[db][rg] = load_b128_device(src + db * 32 + rg * 8);
+          wait_vmcnt<0>();
+#pragma unroll
+          for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int rg = 0; rg < 4; ++rg) settle(part[db][rg]);
+#pragma unroll
+          for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int rg = 0; rg < 4; ++rg)
+#pragma unroll
+              for (int e = 0; e < 4; ++e) o[db][qb][rg * 4 + e] += wgt * part[db][rg][e];
+        }
+      }
+      const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
+      T* dst = static_cast<T*>(p.out) + b * p.out_stride[0] + head * p.out_stride[1] + i * p.out_stride[2];
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {
+          typename M::Vec4 v4;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v4[e] = static_cast<T>(o[db][qb][rg * 4 + e] * inv);
+          *reinterpret_cast<typename M::Vec4*>(dst + db * 32 + rg * 8 + 4 * lh) = v4;
+        }
     }
   }
 #ifdef FTA_DBG_TIMING

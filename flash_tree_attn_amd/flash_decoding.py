@@ -33,6 +33,19 @@ class FtaAssertionError(ValueError, AssertionError):
 
 _ASSERT_STATUSES = {-2, -3, -4, -5}
 _cu_count = {}
+_counters = {}
+
+
+def _counters_for(device: torch.device, stream: int, elems: int) -> torch.Tensor:
+    """Zeroed int32 counters for the single-launch merge. The kernel leaves them zero
+    again, so one buffer per (device, stream) serves every call issued on that stream;
+    calls on different streams may overlap in time and get buffers of their own."""
+    key = (device.index, stream)
+    buf = _counters.get(key)
+    if buf is None or buf.numel() < elems:
+        buf = torch.zeros(max(elems, 4096), dtype=torch.int32, device=device)
+        _counters[key] = buf
+    return buf
 
 
 def _check(status: int) -> None:
@@ -158,13 +171,28 @@ class PreparedCall:
         self._lib = _lib.load()
         self._ref = C.byref(args)
 
-    def _launch(self, fn):
+    def _launch(self, fn, single_launch=False):
         with torch.cuda.device(self._device):
             stream = torch.cuda.current_stream(self._device).cuda_stream
+            if single_launch and self.plan.counter_elems > 0:
+                buf = _counters_for(self._device, stream, self.plan.counter_elems)
+                self.args.counters, self.args.counter_elems = buf.data_ptr(), buf.numel()
+            else:
+                self.args.counters, self.args.counter_elems = None, 0
             _check(fn(self._ref, C.c_void_p(stream)))
         return self.output
 
     def run(self):
+        """The whole path: one launch where the plan advises the merge inside stage 1
+        (few splits), else stage 1 + stage 2."""
+        return self._launch(self._lib.fta_decode, single_launch=bool(self.plan.single_launch))
+
+    def run_single_launch(self):
+        """The whole path in one launch wherever the plan has counters, advised or not."""
+        return self._launch(self._lib.fta_decode, single_launch=True)
+
+    def run_two_launches(self):
+        """The whole path as stage 1 + stage 2 kernels (what a caller without counters gets)."""
         return self._launch(self._lib.fta_decode)
 
     def run_stage1(self):

@@ -20,7 +20,7 @@
 extern "C" {
 #endif
 
-#define FTA_ABI_VERSION 1
+#define FTA_ABI_VERSION 2
 
 typedef enum fta_status {
   FTA_OK = 0,
@@ -60,6 +60,14 @@ typedef enum fta_kernel {
  *   mid_o     float32 [bsz, num_q_heads, mid_splits, q_len, head_dim]  (flash_tree_attn.py:276-279)
  *   mid_lse   float32 [bsz, num_q_heads, mid_splits, q_len]            (flash_tree_attn.py:280-281)
  * mid_o / mid_lse are scratch; they may be NULL when the plan has num_splits == 1.
+ *   counters  int32 [counter_elems], optional. When given (and the plan reports
+ *             counter_elems > 0), fta_decode runs ONE launch: the workgroup that
+ *             finishes a sequence's last split merges the partials itself, which
+ *             replaces the second kernel of flash_tree_attn.py:339-365 and the gap
+ *             between the two launches. Contract: all zero on entry; the kernel leaves
+ *             them all zero again, so one buffer zeroed once serves every later call on
+ *             the same stream; calls that may overlap in time need buffers of their
+ *             own. NULL keeps the two-launch path.
  */
 typedef struct fta_args {
   const void* q;
@@ -72,6 +80,7 @@ typedef struct fta_args {
   void* out;
   float* mid_o;
   float* mid_lse;
+  int32_t* counters;
 
   int32_t bsz;
   int32_t num_q_heads;
@@ -88,6 +97,7 @@ typedef struct fta_args {
   int32_t len_dtype;        /* fta_len_dtype of kv_seq_len */
   int32_t force_splits;     /* 0 = heuristic; >0 pins the split count (tuning, tests) */
   int32_t force_kernel;     /* -1 = heuristic; else an fta_kernel */
+  int32_t counter_elems;    /* int32 elements behind `counters`, 0 when it is NULL */
   float sm_scale;
 
   int64_t q_stride[3];      /* batch, head, row */
@@ -110,6 +120,10 @@ typedef struct fta_plan_out {
   int32_t rows_per_wg;    /* query rows one workgroup holds */
   int32_t row_blocks;     /* ceil(rows_per_group / rows_per_wg) */
   int32_t num_workgroups; /* stage-1 grid size */
+  int32_t counter_elems;  /* int32 counters the single-launch path needs; 0 = this plan has no such path */
+  int32_t single_launch;  /* 1 where the single-launch path is expected to be the faster one (two splits, one
+                             round of workgroups: the last workgroup of a sequence merges alone, which does
+                             not pay for more) */
   int32_t reserved;
   int64_t mid_o_elems;    /* float32 elements a dense mid_o for this plan needs */
   int64_t mid_lse_elems;
@@ -133,7 +147,8 @@ int fta_validate(const fta_args* args);
 int fta_plan(const fta_args* args, int num_cus, fta_plan_out* plan);
 
 /* Runs the whole path (stage 1 with the tree block folded in, then the LSE merge
- * when the plan has more than one split) on `hip_stream` (a hipStream_t; NULL is
+ * when the plan has more than one split: inside the same launch when `counters`
+ * is given, as a second kernel otherwise) on `hip_stream` (a hipStream_t; NULL is
  * the default stream). Replaces flash_tree_attn.py:293-376. Asynchronous. */
 int fta_decode(const fta_args* args, void* hip_stream);
 

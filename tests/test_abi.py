@@ -4,6 +4,7 @@ and plans splits sensibly. No kernel is launched here."""
 import ctypes as C
 import os
 import re
+import subprocess
 
 import pytest
 
@@ -50,10 +51,27 @@ def test_header_symbols_exported(fta_lib):
     assert int(re.search(r"#define FTA_ABI_VERSION (\d+)", header).group(1)) == _lib.ABI_VERSION
 
 
-def test_struct_layout_matches_header(fta_lib):
-    # 10 pointers, 15 int32 + 1 float, 9 stride arrays (8 of 3 + 1 of 4 int64)
-    assert C.sizeof(_lib.FtaArgs) == 10 * 8 + 16 * 4 + (8 * 3 + 4) * 8
-    assert C.sizeof(_lib.FtaPlanOut) == 8 * 4 + 2 * 8
+def test_struct_layout_matches_header(fta_lib, tmp_path):
+    # 11 pointers, 16 int32 + 1 float (padded to 8), 9 stride arrays (8 of 3 + 1 of 4 int64)
+    assert C.sizeof(_lib.FtaArgs) == 11 * 8 + 18 * 4 + (8 * 3 + 4) * 8
+    assert C.sizeof(_lib.FtaPlanOut) == 10 * 4 + 2 * 8
+    # ... and field by field against what a C compiler makes of include/fta.h
+    fields = [n for n, _ in _lib.FtaArgs._fields_]
+    plan_fields = [n for n, _ in _lib.FtaPlanOut._fields_]
+    src = tmp_path / "layout.c"
+    lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "fta.h"', 'int main(void) {',
+             '  printf("%zu %zu\\n", sizeof(fta_args), sizeof(fta_plan_out));']
+    lines += [f'  printf("%zu\\n", offsetof(fta_args, {n}));' for n in fields]
+    lines += [f'  printf("%zu\\n", offsetof(fta_plan_out, {n}));' for n in plan_fields]
+    lines += ['  return 0;', '}']
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
+    assert [int(out[0]), int(out[1])] == [C.sizeof(_lib.FtaArgs), C.sizeof(_lib.FtaPlanOut)]
+    offs = [int(v) for v in out[2:]]
+    assert offs[:len(fields)] == [getattr(_lib.FtaArgs, n).offset for n in fields]
+    assert offs[len(fields):] == [getattr(_lib.FtaPlanOut, n).offset for n in plan_fields]
 
 
 def test_strerror(fta_lib):
@@ -147,6 +165,10 @@ def test_plan_properties(fta_lib, kw, cus):
         assert pl.mid_o_elems == 0 and pl.mid_lse_elems == 0
     mfma_ok = a.dtype in (_lib.FTA_F16, _lib.FTA_BF16) and a.head_dim in (64, 128) and pl.rows_per_group >= 16
     assert pl.kernel == (_lib.KERNEL_MFMA if mfma_ok else _lib.KERNEL_SHUFFLE)
+    # one counter per (sequence, unit, row block) where the merge can run inside stage 1
+    fusable = pl.num_splits > 1 and pl.kernel == _lib.KERNEL_MFMA
+    assert pl.counter_elems == (pl.num_workgroups // pl.num_splits if fusable else 0)
+    assert pl.single_launch == int(fusable and pl.num_splits <= 2 and pl.num_workgroups <= cus)
 
 
 def test_plan_headline_shape_fills_the_gpu(fta_lib):

@@ -301,6 +301,37 @@ def test_ragged_batch_dispatch_order(bsz, splits):
     check(run(x, _force_splits=splits, _force_kernel=_lib.KERNEL_SHUFFLE), ref, torch.float16)
 
 
+@pytest.mark.parametrize("shape", [
+    # bsz hq hkv  L   D   tmax  lens                      splits
+    (8, 32, 8, 64, 128, 2048, None, 4),                    # headline layout: 256 rows, 4 splits
+    (5, 16, 2, 16, 128, 1500, [1500, 700, 64, 0, 1499], 5),  # 128 rows, ragged: 1..5 live splits
+    (3, 12, 3, 40, 64, 900, [900, 450, 1], 3),             # D 64, padded row block
+    (2, 16, 2, 40, 128, 700, [700, 300], 4),               # two row blocks per group
+])
+def test_single_launch_merge_matches_two_launches(shape):
+    """With counters, the workgroup that finishes a sequence last merges the partials
+    inside stage 1. Same result as stage 1 + stage 2, on repeated calls (the counters
+    must be left zero), and the counters really are zero afterwards."""
+    from flash_tree_attn_amd import flash_decoding as fd
+    bsz, hq, hkv, L, D, tmax, lens, splits = shape
+    x = make(61, bsz, hq, hkv, L, D, tmax, torch.bfloat16, lens if lens is not None else [tmax] * bsz)
+    ref = oracle(x)
+    pc = fd.prepare(x["q"], x["k_cache"], x["v_cache"], x["current_k"], x["current_v"], x["mask"], x["kv_seq_len"],
+                 64, None, None, None, None, None, x["kv_group_num"], _force_splits=splits)
+    assert pc.plan.kernel == _lib.KERNEL_MFMA and pc.plan.num_splits == splits and pc.plan.counter_elems > 0
+    two = pc.run_two_launches().clone()
+    check(two, ref, torch.bfloat16)
+    for _ in range(3):
+        pc.output.fill_(float("nan"))
+        one = pc.run_single_launch().clone()
+        check(one, ref, torch.bfloat16)
+        torch.testing.assert_close(one.float(), two.float(), atol=1e-5, rtol=2 ** -7)
+    torch.cuda.synchronize()
+    stream = torch.cuda.current_stream().cuda_stream
+    buf = fd._counters[(x["q"].device.index, stream)]
+    assert int(buf.abs().sum()) == 0
+
+
 # ---------------------------------------------------------------- size-independent properties
 def test_properties_at_headline_size():
     cfg = CONFIGS["cfg3_gqa_8b_bf16"]
