@@ -82,19 +82,22 @@ __device__ __forceinline__ WorkItem decode_work(const KernelParams& p, int id) {
 // first every full chunk (all equal work; sequence-major), then the last chunk of every
 // sequence (partial chunk + tree block) in descending size; what remains of the grid has
 // nothing to do. No host look at the lengths and no atomics: every workgroup recomputes
-// the order from the bsz lengths in one LDS pass. Batches of one sequence or beyond
+// the order from the bsz lengths in one LDS pass (and gets its sequence's clamped length
+// back with it). Batches of one sequence or beyond
 // kMaxOrderedBatch keep the identity order. Returns false if the item is empty. Must be
 // called by all threads of the block.
 constexpr int kMaxOrderedBatch = 256;
-__device__ __forceinline__ bool item_by_order(const KernelParams& p, int k, int* batch, int* split) {
+__device__ __forceinline__ bool item_by_order(const KernelParams& p, int k, int* batch, int* split, int* len) {
   if (p.bsz == 1 || p.bsz > kMaxOrderedBatch) {
     *batch = k / p.num_splits;
     *split = k % p.num_splits;
+    const int64_t v = load_len(p.lens, p.len_is_i64, *batch);
+    *len = static_cast<int>(v < 0 ? 0 : (v > p.cache_len ? p.cache_len : v));
     return true;
   }
   __shared__ int s_nsp[kMaxOrderedBatch];
   __shared__ int s_tail[kMaxOrderedBatch];
-  __shared__ int s_pick[2];
+  __shared__ int s_pick[3];
   const int t = threadIdx.x;
   for (int i = t; i < p.bsz; i += blockDim.x) {
     const int64_t v = load_len(p.lens, p.len_is_i64, i);
@@ -114,17 +117,17 @@ __device__ __forceinline__ bool item_by_order(const KernelParams& p, int k, int*
       before += j < i ? f : 0;
       rank += (s_tail[j] > mine) || (s_tail[j] == mine && j < i);
     }
-    if (k >= before && k < before + s_nsp[i] - 1) {
+    const bool full = k >= before && k < before + s_nsp[i] - 1;
+    if (full || k - total == rank) {
       s_pick[0] = i;
-      s_pick[1] = k - before;
-    } else if (k - total == rank) {
-      s_pick[0] = i;
-      s_pick[1] = s_nsp[i] - 1;
+      s_pick[1] = full ? k - before : s_nsp[i] - 1;
+      s_pick[2] = mine + (s_nsp[i] - 1) * p.chunk;   // the (clamped) length, so that callers need not load it again
     }
   }
   __syncthreads();
   *batch = __builtin_amdgcn_readfirstlane(s_pick[0]);  // uniform: keep them in scalar registers
   *split = __builtin_amdgcn_readfirstlane(s_pick[1]);
+  *len = __builtin_amdgcn_readfirstlane(s_pick[2]);
   return *batch >= 0;
 }
 

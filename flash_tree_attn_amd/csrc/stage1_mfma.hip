@@ -44,6 +44,12 @@ template <> struct Mfma<__bf16> {
   static __device__ __forceinline__ f32x16 mma(Vec8 a, Vec8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
+  // acc + v[0] + v[1]: one instruction sums a packed pair (and sums the ROUNDED values,
+  // the very weights the P.V product applies)
+  static __device__ __forceinline__ float add_pair(Vec2 v, float acc) {
+    const Vec2 ones = {static_cast<__bf16>(1.f), static_cast<__bf16>(1.f)};
+    return __builtin_amdgcn_fdot2_f32_bf16(v, ones, acc, false);
+  }
 };
 template <> struct Mfma<_Float16> {
   using Vec8 = f16x8;
@@ -51,6 +57,10 @@ template <> struct Mfma<_Float16> {
   using Vec2 = f16x2;
   static __device__ __forceinline__ f32x16 mma(Vec8 a, Vec8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float add_pair(Vec2 v, float acc) {
+    const Vec2 ones = {static_cast<_Float16>(1.f), static_cast<_Float16>(1.f)};
+    return __builtin_amdgcn_fdot2(v, ones, acc, false);
   }
 };
 
@@ -154,14 +164,14 @@ __device__ __forceinline__ void static_for(F&& f) {
 
 // NSK >= 2: K of tile t+1 is read during iteration t and must have been requested an
 // iteration earlier.
-template <typename T, int D, int QB, int NW, int NSK>
+template <typename T, int D, int QB, int NW, int NSK, bool PIPE>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(QB == 1 ? 2 : 1, QB == 1 ? 2 : 1)))
 stage1_mfma_kernel(const KernelParams p) {
   using M = Mfma<T>;
   using Vec8 = typename M::Vec8;
   using TL = TileLayout<D>;
   static_assert(NSK >= 2, "K ring too shallow");
-  constexpr int NSV = NSK + 2;                       // V of a tile is read one iteration after its K
+  constexpr int NSV = PIPE ? NSK + 2 : NSK;          // pipelined: V of a tile is read one iteration after its K
   constexpr int KS = D / 16;                         // k-steps of the QK product
   constexpr int DB = D / 32;                         // head_dim blocks of the PV product
   constexpr int RPB = TL::kRowsPerBlock;
@@ -182,10 +192,8 @@ stage1_mfma_kernel(const KernelParams p) {
   FTA_STAMP();
 
   const WorkItem w = decode_work(p, blockIdx.x);
-  int b, split;
-  if (!item_by_order(p, w.item, &b, &split)) return;
-  int64_t t64 = load_len(p.lens, p.len_is_i64, b);
-  const int T_b = static_cast<int>(t64 < 0 ? 0 : (t64 > p.cache_len ? p.cache_len : t64));
+  int b, split, T_b;
+  if (!item_by_order(p, w.item, &b, &split, &T_b)) return;
   const int S_b = splits_for(T_b, p.chunk, p.num_splits);
   if (split >= S_b) return;
   const int kv_start = split * p.chunk;
@@ -617,10 +625,9 @@ stage1_mfma_kernel(const KernelParams p) {
             const int x = 2 * j, kb = x / 16, r = x % 16;
             const float p0 = fast_exp2(__builtin_fmaf(s_in[kb][qb][r], c, -m_new[qb]));
             const float p1 = fast_exp2(__builtin_fmaf(s_in[kb][qb][r + 1], c, -m_new[qb]));
-            ps0[qb] += p0;
-            ps1[qb] += p1;
             const f32x2 pv = {p0, p1};
             const auto pr = __builtin_convertvector(pv, typename M::Vec2);
+            if (j & 1) ps1[qb] = M::add_pair(pr, ps1[qb]); else ps0[qb] = M::add_pair(pr, ps0[qb]);
             p_out[qb][kb * 2 + (r >= 8)][r % 8] = pr[0];
             p_out[qb][kb * 2 + (r >= 8)][r % 8 + 1] = pr[1];
           }
@@ -660,88 +667,109 @@ stage1_mfma_kernel(const KernelParams p) {
   };
 
   float mask_vals[QB][2][16];
-  // phase A: the tree tiles, one complete step each (scores, masked softmax, P.V twice)
   const int c0 = tree_tiles;   // first cache tile
-  for (int u = 0; u < tree_tiles; ++u) {
-    sync_point(u, u, u);
-    if (!wave_active) continue;
-    load_mask(u * kKeyTile, mask_vals);   // in flight while the scores are computed
-    qk_tile(u, sB);
-    softmax_tile(std::true_type{}, sB, pA, true, u * kKeyTile, L, mask_vals);
-    pv_with_residue(u, true, sB);
-  }
-  FTA_STAMP();
+  if constexpr (!PIPE) {
+    // Plain variant: every tile runs scores -> softmax -> P.V back to back, with the next
+    // tile in flight. Its small LDS footprint lets two workgroups share a CU; their
+    // phases (matrix, vector, waiting, prologue, epilogue) overlap each other instead
+    // of being interleaved by hand.
+    for (int t = 0; t < ntiles; ++t) {
+      sync_point(t, t, t);
+      if (!wave_active) continue;
+      const bool tree = t < tree_tiles;
+      const bool masked = tree || t - c0 >= full_tiles;
+      const int key0 = tree ? t * kKeyTile : kv_start + (t - c0) * kKeyTile;
+      if (tree) load_mask(key0, mask_vals);   // in flight while the scores are computed
+      qk_tile(t, sB);
+      if (masked) softmax_tile(std::true_type{}, sB, pA, tree, key0, tree ? L : kv_end, mask_vals);
+      else softmax_tile(std::false_type{}, sB, pA, false, key0, kv_end, mask_vals);
+      pv_with_residue(t, masked, sB);
+    }
+    if (!wave_active) return;
+  } else {
+    // phase A: the tree tiles, one complete step each (scores, masked softmax, P.V twice)
+    FTA_STAMP();
+    for (int u = 0; u < tree_tiles; ++u) {
+      sync_point(u, u, u);
+      if (!wave_active) continue;
+      load_mask(u * kKeyTile, mask_vals);   // in flight while the scores are computed
+      qk_tile(u, sB);
+      softmax_tile(std::true_type{}, sB, pA, true, u * kKeyTile, L, mask_vals);
+      pv_with_residue(u, true, sB);
+    }
+    FTA_STAMP();
 
-  // phase B: fused iterations over the full cache tiles that have a successor
-  const int fused_cnt = cache_tiles >= 1 ? min(full_tiles, cache_tiles - 1) : 0;
-  int t = c0;
-  bool cur_in_B = false;   // which buffer pair holds the current scores / previous P
-  if (cache_tiles >= 1) {
-    sync_point(c0, c0, c0);
-    if (wave_active) qk_tile(c0, sA);
-  }
-  if (fused_cnt >= 1) {
-    sync_point(c0 + 1, c0 + 1, c0);
-    if (wave_active) fused(std::false_type{}, c0, sA, sB, pB, pA);
-    t = c0 + 1;
-    cur_in_B = true;
-    for (; t + 1 < c0 + fused_cnt; t += 2) {
-      sync_point(t + 1, t + 1, max(c0, t - 1));
-      if (wave_active) {
-        apply_rescale();
-        fused(std::true_type{}, t, sB, sA, pA, pB);
+    // phase B: fused iterations over the full cache tiles that have a successor
+    const int fused_cnt = cache_tiles >= 1 ? min(full_tiles, cache_tiles - 1) : 0;
+    int t = c0;
+    bool cur_in_B = false;   // which buffer pair holds the current scores / previous P
+    if (cache_tiles >= 1) {
+      sync_point(c0, c0, c0);
+      if (wave_active) qk_tile(c0, sA);
+    }
+    if (fused_cnt >= 1) {
+      sync_point(c0 + 1, c0 + 1, c0);
+      if (wave_active) fused(std::false_type{}, c0, sA, sB, pB, pA);
+      t = c0 + 1;
+      cur_in_B = true;
+      for (; t + 1 < c0 + fused_cnt; t += 2) {
+        sync_point(t + 1, t + 1, max(c0, t - 1));
+        if (wave_active) {
+          apply_rescale();
+          fused(std::true_type{}, t, sB, sA, pA, pB);
+        }
+        sync_point(t + 2, t + 2, max(c0, t));
+        if (wave_active) {
+          apply_rescale();
+          fused(std::true_type{}, t + 1, sA, sB, pB, pA);
+        }
       }
-      sync_point(t + 2, t + 2, max(c0, t));
-      if (wave_active) {
-        apply_rescale();
-        fused(std::true_type{}, t + 1, sA, sB, pB, pA);
+      if (t < c0 + fused_cnt) {
+        sync_point(t + 1, t + 1, max(c0, t - 1));
+        if (wave_active) {
+          apply_rescale();
+          fused(std::true_type{}, t, sB, sA, pA, pB);
+        }
+        ++t;
+        cur_in_B = false;
       }
     }
-    if (t < c0 + fused_cnt) {
-      sync_point(t + 1, t + 1, max(c0, t - 1));
-      if (wave_active) {
-        apply_rescale();
-        fused(std::true_type{}, t, sB, sA, pA, pB);
-      }
-      ++t;
-      cur_in_B = false;
+    FTA_STAMP();
+    // canonical roles for the tail: current scores in sB, previous P in pA
+    bool pv_pending = fused_cnt >= 1;   // P of tile t-1 has not been multiplied yet
+    bool prv_masked = false;
+    if (!cur_in_B) {
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) sB[kb][qb] = sA[kb][qb];
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) pA[qb][kk] = pB[qb][kk];
     }
-  }
-  FTA_STAMP();
-  // canonical roles for the tail: current scores in sB, previous P in pA
-  bool pv_pending = fused_cnt >= 1;   // P of tile t-1 has not been multiplied yet
-  bool prv_masked = false;
-  if (!cur_in_B) {
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-      for (int qb = 0; qb < QB; ++qb) sB[kb][qb] = sA[kb][qb];
-#pragma unroll
-    for (int qb = 0; qb < QB; ++qb)
-#pragma unroll
-      for (int kk = 0; kk < 4; ++kk) pA[qb][kk] = pB[qb][kk];
-  }
 
-  // phase C: the last cache tiles of the split, step by step (the last one may be ragged)
-  for (; t < ntiles; ++t) {
-    sync_point(t + 1 < ntiles ? t + 1 : -1, t + 1, max(c0, t - 1));
-    if (!wave_active) continue;
-    const bool masked = t - c0 >= full_tiles;
-    if (pv_pending) pv_with_residue(t - 1, prv_masked, sA);
-    if (masked) softmax_tile(std::true_type{}, sB, pA, false, kv_start + (t - c0) * kKeyTile, kv_end, mask_vals);
-    else softmax_tile(std::false_type{}, sB, pA, false, kv_start + (t - c0) * kKeyTile, kv_end, mask_vals);
-    // a masked tile leaves the rounding residue of P in sB: park it in sA, the scores of
-    // tile t+1 go to sB
+    // phase C: the last cache tiles of the split, step by step (the last one may be ragged)
+    for (; t < ntiles; ++t) {
+      sync_point(t + 1 < ntiles ? t + 1 : -1, t + 1, max(c0, t - 1));
+      if (!wave_active) continue;
+      const bool masked = t - c0 >= full_tiles;
+      if (pv_pending) pv_with_residue(t - 1, prv_masked, sA);
+      if (masked) softmax_tile(std::true_type{}, sB, pA, false, kv_start + (t - c0) * kKeyTile, kv_end, mask_vals);
+      else softmax_tile(std::false_type{}, sB, pA, false, kv_start + (t - c0) * kKeyTile, kv_end, mask_vals);
+      // a masked tile leaves the rounding residue of P in sB: park it in sA, the scores of
+      // tile t+1 go to sB
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
+      for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-      for (int qb = 0; qb < QB; ++qb) sA[kb][qb] = sB[kb][qb];
-    if (t + 1 < ntiles) qk_tile(t + 1, sB);
-    pv_pending = true;
-    prv_masked = masked;
+        for (int qb = 0; qb < QB; ++qb) sA[kb][qb] = sB[kb][qb];
+      if (t + 1 < ntiles) qk_tile(t + 1, sB);
+      pv_pending = true;
+      prv_masked = masked;
+    }
+    if (!wave_active) return;
+    if (pv_pending) pv_with_residue(ntiles - 1, prv_masked, sA);
   }
-  if (!wave_active) return;
-  if (pv_pending) pv_with_residue(ntiles - 1, prv_masked, sA);
   FTA_STAMP();
 
   // ---- epilogue
@@ -884,11 +912,11 @@ stage1_mfma_kernel(const KernelParams p) {
 #endif
 }
 
-template <typename T, int D, int QB, int NW, int NS>
+template <typename T, int D, int QB, int NW, int NS, bool PIPE>
 int launch(const KernelParams& p, hipStream_t stream) {
-  constexpr int kSmem = (2 * NS + 2) * TileLayout<D>::kTileBytes;  // K ring of NS stages + V ring of NS + 2
+  constexpr int kSmem = (PIPE ? 2 * NS + 2 : 2 * NS) * TileLayout<D>::kTileBytes;  // K ring of NS stages + V ring of NS (+ 2)
   static_assert(kSmem <= 160 * 1024, "LDS budget");
-  auto kern = stage1_mfma_kernel<T, D, QB, NW, NS>;
+  auto kern = stage1_mfma_kernel<T, D, QB, NW, NS, PIPE>;
   if (kSmem > 64 * 1024) {
     // Raising the dynamic-LDS limit is a driver call: once per kernel and device, not per launch.
     static thread_local int configured_device = -1;
@@ -908,12 +936,12 @@ int launch(const KernelParams& p, hipStream_t stream) {
 
 template <typename T>
 int launch_t(const KernelParams& p, int head_dim, hipStream_t stream) {
-  if (p.rows_per_wg == 256) {  // 8 waves, one workgroup per CU, K ring 3 / V ring 5
-    if (head_dim == 128) return launch<T, 128, 1, 8, 3>(p, stream);
-    if (head_dim == 64) return launch<T, 64, 1, 8, 3>(p, stream);
-  } else if (p.rows_per_wg == 128) {  // 4 waves, same rings
-    if (head_dim == 128) return launch<T, 128, 1, 4, 3>(p, stream);
-    if (head_dim == 64) return launch<T, 64, 1, 4, 3>(p, stream);
+  if (p.rows_per_wg == 256) {  // 8 waves, pipelined, one workgroup per CU, K ring 3 / V ring 5
+    if (head_dim == 128) return launch<T, 128, 1, 8, 3, true>(p, stream);
+    if (head_dim == 64) return launch<T, 64, 1, 8, 3, true>(p, stream);
+  } else if (p.rows_per_wg == 128) {  // 4 waves, plain, two workgroups per CU, K and V rings of 2
+    if (head_dim == 128) return launch<T, 128, 1, 4, 2, false>(p, stream);
+    if (head_dim == 64) return launch<T, 64, 1, 4, 2, false>(p, stream);
   }
   return FTA_ERR_UNSUPPORTED;
 }

@@ -41,10 +41,8 @@ __global__ void __launch_bounds__(256) stage1_shuffle_kernel(const KernelParams 
   float* Ps = reinterpret_cast<float*>(smem + S::kKBytes + S::kVBytes + S::kQBytes);
 
   const WorkItem w = decode_work(p, blockIdx.x);
-  int b, split;
-  if (!item_by_order(p, w.item, &b, &split)) return;
-  int64_t t64 = load_len(p.lens, p.len_is_i64, b);
-  const int T_b = static_cast<int>(t64 < 0 ? 0 : (t64 > p.cache_len ? p.cache_len : t64));
+  int b, split, T_b;
+  if (!item_by_order(p, w.item, &b, &split, &T_b)) return;
   const int S_b = splits_for(T_b, p.chunk, p.num_splits);
   if (split >= S_b) return;
   const int kv_start = split * p.chunk;
