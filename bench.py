@@ -30,6 +30,7 @@ def parse():
     ap.add_argument("--config", default="cfg3_gqa_8b_bf16", help="workload name (flash_tree_attn_amd.synthetic.CONFIGS)")
     ap.add_argument("--kv-sets", type=int, default=0, help="independent KV caches to rotate over (0 = enough for >1 GiB)")
     ap.add_argument("--splits", type=int, default=0, help="pin the split count (0 = heuristic)")
+    ap.add_argument("--packed-mask", action="store_true", help="pass the tree mask as packed bit words instead of float32")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run plain device copies of a known size (reference point for rocprofv3 FETCH_SIZE / WRITE_SIZE)")
@@ -117,11 +118,15 @@ def main():
     small = kv_bytes * kv_sets < (64 << 20)
     x = make_inputs(cfg, seed=0, device=dev, gen_device="cpu" if small else dev, kv_sets=kv_sets)
 
-    calls = [prepare(x["q"], kc, vc, x["current_k"], x["current_v"], x["mask"], x["kv_seq_len"], cfg.block_size,
+    mask_arg = x["mask"]
+    if args.packed_mask:
+        from flash_tree_attn_amd.tree_mask import pack_mask
+        mask_arg = pack_mask(x["mask"])
+    calls = [prepare(x["q"], kc, vc, x["current_k"], x["current_v"], mask_arg, x["kv_seq_len"], cfg.block_size,
                      None, None, None, None, x["sm_scale"], cfg.kv_group_num, _force_splits=args.splits)
              for kc, vc in zip(x["k_caches"], x["v_caches"])]
     plan = calls[0].plan
-    nbytes = algorithmic_bytes(cfg, x["kv_seq_len"].cpu(), x["mask"])
+    nbytes = algorithmic_bytes(cfg, x["kv_seq_len"].cpu(), mask_arg)
     nflops = flops(cfg, x["kv_seq_len"].cpu())
 
     # quick self-check of the measured path against the oracle on one sequence
@@ -165,7 +170,7 @@ def main():
         "data": "synthetic (seed 0, N(0,1) q/k/v, random tree mask), inputs resident in HBM",
         "config": {"workload": cfg.name, "bsz": cfg.bsz, "q_heads": cfg.num_heads, "kv_heads": cfg.num_kv_heads,
                    "head_dim": cfg.head_dim, "q_len": cfg.q_len, "cache_len": cfg.cache_len, "lengths": cfg.lengths,
-                   "block_size": cfg.block_size, "kv_sets_rotated": kv_sets, "num_splits": plan.num_splits,
+                   "block_size": cfg.block_size, "mask": "packed u64" if args.packed_mask else "additive f32", "kv_sets_rotated": kv_sets, "num_splits": plan.num_splits,
                    "chunk": plan.chunk, "stage1_kernel": "mfma" if plan.kernel == _lib.KERNEL_MFMA else "shuffle",
                    "stage1_workgroups": plan.num_workgroups, "algorithmic_bytes": nbytes, "flops": nflops},
         "tflops": nflops / (ms * 1e-3) / 1e12,

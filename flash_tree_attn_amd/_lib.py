@@ -10,6 +10,7 @@ LIB_PATH = os.path.join(HERE, "libfta.so")
 ABI_VERSION = 2
 FTA_F32, FTA_F16, FTA_BF16 = 0, 1, 2
 FTA_I32, FTA_I64 = 0, 1
+MASK_ADDITIVE_F32, MASK_PACKED_U64 = 0, 1
 KERNEL_SHUFFLE, KERNEL_MFMA = 0, 1
 
 EXPORTED_SYMBOLS = (
@@ -31,7 +32,7 @@ class FtaArgs(C.Structure):
         ("q_len", C.c_int32), ("head_dim", C.c_int32), ("cache_len", C.c_int32), ("v_cache_len", C.c_int32),
         ("block_size", C.c_int32), ("max_seq_len_hint", C.c_int32), ("mid_splits", C.c_int32),
         ("dtype", C.c_int32), ("len_dtype", C.c_int32), ("force_splits", C.c_int32), ("force_kernel", C.c_int32),
-        ("counter_elems", C.c_int32), ("sm_scale", C.c_float),
+        ("counter_elems", C.c_int32), ("mask_kind", C.c_int32), ("sm_scale", C.c_float),
         ("q_stride", C.c_int64 * 3), ("k_stride", C.c_int64 * 3), ("v_stride", C.c_int64 * 3),
         ("ck_stride", C.c_int64 * 3), ("cv_stride", C.c_int64 * 3), ("mask_stride", C.c_int64 * 3),
         ("out_stride", C.c_int64 * 3), ("mid_o_stride", C.c_int64 * 4), ("mid_lse_stride", C.c_int64 * 3),

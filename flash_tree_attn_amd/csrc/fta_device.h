@@ -31,6 +31,17 @@ __device__ __forceinline__ int64_t load_len(const void* lens, int is_i64, int b)
   return is_i64 ? static_cast<const int64_t*>(lens)[b] : static_cast<int64_t>(static_cast<const int32_t*>(lens)[b]);
 }
 
+// Additive mask value of tree key j for the mask row that starts at element `row_start`
+// (in elements of the mask's type): the float itself, or 0 / -inf from bit j of a
+// packed row.
+__device__ __forceinline__ float tree_mask_value(const KernelParams& p, int64_t row_start, int j) {
+  if (p.mask_packed) {
+    const uint64_t w = static_cast<const uint64_t*>(p.mask)[row_start + (j >> 6)];
+    return (w >> (j & 63)) & 1 ? 0.f : neg_inf();
+  }
+  return static_cast<const float*>(p.mask)[row_start + j];
+}
+
 // Splits that hold data for a sequence of `t` cached keys: ceil(t / chunk), at
 // least one (the tree block always needs a home), at most the grid extent.
 __device__ __forceinline__ int splits_for(int t, int chunk, int num_splits) {

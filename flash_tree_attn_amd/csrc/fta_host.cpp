@@ -44,6 +44,7 @@ int validate(const fta_args& a) {
     return FTA_ERR_NULL_POINTER;
   if (a.dtype != FTA_F32 && a.dtype != FTA_F16 && a.dtype != FTA_BF16) return FTA_ERR_DTYPE;
   if (a.len_dtype != FTA_I32 && a.len_dtype != FTA_I64) return FTA_ERR_DTYPE;
+  if (a.mask_kind != FTA_MASK_ADDITIVE_F32 && a.mask_kind != FTA_MASK_PACKED_U64) return FTA_ERR_DTYPE;
   if (a.head_dim != 32 && a.head_dim != 64 && a.head_dim != 128 && a.head_dim != 256) return FTA_ERR_HEAD_DIM;
   if (a.cache_len != a.v_cache_len) return FTA_ERR_CACHE_LEN_MISMATCH;
   if (a.block_size != 16 && a.block_size != 32 && a.block_size != 64 && a.block_size != 128)
@@ -68,6 +69,7 @@ int validate(const fta_args& a) {
     if (reinterpret_cast<uintptr_t>(ptr) % 16 != 0) return FTA_ERR_STRIDE;
   for (int i = 0; i < 3; ++i)
     if (a.mask_stride[i] < 0) return FTA_ERR_STRIDE;
+  if (reinterpret_cast<uintptr_t>(a.mask) % (a.mask_kind == FTA_MASK_PACKED_U64 ? 8 : 4) != 0) return FTA_ERR_STRIDE;
   return FTA_OK;
 }
 
@@ -201,7 +203,7 @@ int fta_plan(const fta_args* args, int num_cus, fta_plan_out* plan) {
   alignas(16) static const char aligned_dummy[16] = {0};
   const void* d = aligned_dummy;
   a.q = a.k_cache = a.v_cache = a.cur_k = a.cur_v = a.kv_seq_len = d;
-  a.mask = reinterpret_cast<const float*>(d);
+  a.mask = d;
   a.out = const_cast<void*>(d);
   if (int st = fta::validate(a)) return st;
   return fta::plan(a, num_cus, plan);
@@ -253,7 +255,8 @@ int decode_impl(const fta_args* args, void* hip_stream, int stages) {
   p.cur_group = a.num_q_heads / a.cur_heads;
   p.rows = pl.rows_per_group; p.rows_per_wg = pl.rows_per_wg; p.row_blocks = pl.row_blocks;
   p.len_is_i64 = a.len_dtype == FTA_I64;
-  p.mask_vec4 = reinterpret_cast<uintptr_t>(a.mask) % 16 == 0 && a.mask_stride[0] % 4 == 0 && a.mask_stride[1] % 4 == 0 &&
+  p.mask_packed = a.mask_kind == FTA_MASK_PACKED_U64;
+  p.mask_vec4 = !p.mask_packed && reinterpret_cast<uintptr_t>(a.mask) % 16 == 0 && a.mask_stride[0] % 4 == 0 && a.mask_stride[1] % 4 == 0 &&
                 a.mask_stride[2] % 4 == 0;
   p.scale_log2 = a.sm_scale * fta::kLog2e;
   for (int i = 0; i < 3; ++i) {

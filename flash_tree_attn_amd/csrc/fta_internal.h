@@ -19,7 +19,7 @@ struct KernelParams {
   const void* v;
   const void* ck;
   const void* cv;
-  const float* mask;
+  const void* mask;       // float32 additive values, or uint64 bit words when mask_packed
   const void* lens;
   void* out;
   float* mid_o;
@@ -40,7 +40,8 @@ struct KernelParams {
   int32_t rows_per_wg;
   int32_t row_blocks;
   int32_t len_is_i64;
-  int32_t mask_vec4;      // every mask row starts 16-byte aligned
+  int32_t mask_vec4;      // every (float) mask row starts 16-byte aligned
+  int32_t mask_packed;    // mask holds one bit per (row, tree key): set = attend
   float scale_log2;       // sm_scale * log2(e)
 
   int64_t q_stride[3];

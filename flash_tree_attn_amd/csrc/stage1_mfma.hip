@@ -485,7 +485,20 @@ stage1_mfma_kernel(const KernelParams p) {
   auto load_mask = [&](int key0, float (&mv)[QB][2][16]) __attribute__((always_inline)) {
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
-      const float* mrow = p.mask + b * p.mask_stride[0] + row_head[qb] * p.mask_stride[1] + row_i[qb] * p.mask_stride[2];
+      const int64_t mstart = b * p.mask_stride[0] + row_head[qb] * p.mask_stride[1] + row_i[qb] * p.mask_stride[2];
+      if (p.mask_packed) {
+        // one 64-bit word covers this row's 64 keys of the tile (key0 is a multiple of 64)
+        const uint64_t w = static_cast<const uint64_t*>(p.mask)[mstart + (key0 >> 6)];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int j = kb * 32 + (r >> 2) * 8 + 4 * lh + (r & 3);
+            mv[qb][kb][r] = (w >> j) & 1 ? 0.f : neg_inf();
+          }
+        continue;
+      }
+      const float* mrow = static_cast<const float*>(p.mask) + mstart;
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll

@@ -134,9 +134,8 @@ __global__ void __launch_bounds__(256) stage1_shuffle_kernel(const KernelParams 
     for (int rr = 0; rr < kRowsPerWave; ++rr) {
       float sv = s[rr];
       if (tree && key_ok && row_ok[rr]) {
-        const float mv = p.mask[b * p.mask_stride[0] + row_head[rr] * p.mask_stride[1] +
-                                row_i[rr] * p.mask_stride[2] + (key0 + lane)];
-        sv += mv * kLog2e;
+        const int64_t mrow = b * p.mask_stride[0] + row_head[rr] * p.mask_stride[1] + row_i[rr] * p.mask_stride[2];
+        sv += tree_mask_value(p, mrow, key0 + lane) * kLog2e;
       }
       if (!key_ok) sv = neg_inf();
       const float m_new = fmaxf(m_run[rr], wave_max(sv));

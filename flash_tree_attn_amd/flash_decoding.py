@@ -11,7 +11,8 @@ Differences from the reference that a caller can observe (all deliberate):
 * No host sync: `kv_seq_len.max().item()` (flash_tree_attn.py:272) is not needed;
   `max_seq_len_in_batch` is only a hint that shrinks the grid.
 * fp16, bf16 and fp32 inputs; `current_k/current_v` with num_kv_heads or num_heads
-  heads; any q_len >= 1; `mask` float (additive, flash_tree_attn.py:368) or bool.
+  heads; any q_len >= 1; `mask` float (additive, flash_tree_attn.py:368), bool, or int64
+  bit words from `tree_mask.pack_mask` (8 bytes per row and 64 tree keys).
 * A query row whose every logit is -inf yields zeros (the reference yields NaN).
 There is no CPU or eager fallback: CPU tensors and a missing library raise.
 """
@@ -79,6 +80,17 @@ def _num_cus(device: torch.device) -> int:
 def _prepare_mask(mask: torch.Tensor, bsz: int, hq: int, L: int, device) -> torch.Tensor:
     if mask.device != device:
         raise ValueError("mask must live on the same device as q")
+    if mask.dtype == torch.int64:   # packed bits (tree_mask.pack_mask): [..., L, ceil(L/64)]
+        words = (L + 63) // 64
+        if mask.dim() > 4 or mask.dim() < 2 or mask.size(-1) != words or mask.size(-2) != L:
+            raise ValueError(f"a packed mask must be [..., q_len, ceil(q_len/64)] = [..., {L}, {words}], got {tuple(mask.shape)}")
+        while mask.dim() < 4:
+            mask = mask.unsqueeze(0)
+        try:
+            mask = mask.expand(bsz, hq, L, words)
+        except RuntimeError as e:
+            raise ValueError(f"mask of shape {tuple(mask.shape)} does not broadcast to {(bsz, hq, L, words)}") from e
+        return mask if mask.stride(3) == 1 or words == 1 else mask.contiguous()
     if mask.dtype == torch.bool:
         m = torch.zeros(mask.shape, dtype=torch.float32, device=device)
         m.masked_fill_(~mask, float("-inf"))
@@ -149,6 +161,7 @@ def build_args(q, k_cache, v_cache, current_k, current_v, mask, kv_seq_len, bloc
     a.ck_stride[:] = current_k.stride()[:3]
     a.cv_stride[:] = current_v.stride()[:3]
     a.mask_stride[:] = mask.stride()[:3]
+    a.mask_kind = _lib.MASK_PACKED_U64 if mask.dtype == torch.int64 else _lib.MASK_ADDITIVE_F32
     return a, (q, k_cache, v_cache, current_k, current_v, mask, kv_seq_len)
 
 

@@ -4,7 +4,9 @@ The reference's own generator (flash_tree_attn.py:403-414) draws an unseeded ran
 {1, -inf} matrix that is not a tree; real callers (Medusa / EAGLE style drafts) hold
 a parent array. These helpers turn a parent array into the ADDITIVE mask the op
 consumes (flash_tree_attn.py:368): 0 where column j is an ancestor of, or equal to,
-row i, and -inf elsewhere.
+row i, and -inf elsewhere; or into the PACKED form, one bit per (row, tree key) in
+64-bit words (8 bytes per row and 64 keys instead of 256), which the kernels expand to
+0 / -inf themselves.
 """
 from __future__ import annotations
 
@@ -48,3 +50,37 @@ def additive_mask_from_parents(parents: Sequence[int], device=None, dtype=torch.
     mask = torch.full(anc.shape, float("-inf"), dtype=dtype)
     mask[anc] = 0.0
     return mask.to(device) if device is not None else mask
+
+
+def pack_mask(allowed: torch.Tensor) -> torch.Tensor:
+    """Packs a boolean "may attend" tensor [..., L, L] (or an additive mask: finite =
+    attend) into int64 words [..., L, ceil(L/64)]: bit (j % 64) of word j // 64 of row i
+    is set iff row i attends tree key j. The words are uint64 bit patterns stored in
+    int64 (the dtype torch can index and move); `flash_decoding_attention` takes an int64
+    mask to be this form. Additive values other than 0 / -inf cannot be packed."""
+    if allowed.dtype != torch.bool:
+        finite = torch.isfinite(allowed)
+        if bool(((allowed != 0) & finite).any()):
+            raise ValueError("only 0 / -inf additive masks can be packed")
+        allowed = finite
+    L = allowed.size(-1)
+    if allowed.dim() < 2 or allowed.size(-2) != L:
+        raise ValueError(f"mask must be [..., q_len, q_len], got {tuple(allowed.shape)}")
+    words = (L + 63) // 64
+    pad = words * 64 - L
+    a = torch.nn.functional.pad(allowed, (0, pad)).reshape(*allowed.shape[:-1], words, 64).to(torch.int64)
+    weights = torch.ones(64, dtype=torch.int64, device=allowed.device) << torch.arange(64, device=allowed.device)
+    return (a * weights).sum(-1)   # bit 63 wraps into the sign bit: the intended bit pattern
+
+
+def unpack_mask(packed: torch.Tensor, q_len: int) -> torch.Tensor:
+    """Inverse of pack_mask: boolean [..., q_len, q_len]."""
+    shifts = torch.arange(64, device=packed.device)
+    bits = ((packed.unsqueeze(-1) >> shifts) & 1).bool()
+    return bits.reshape(*packed.shape[:-1], packed.size(-1) * 64)[..., :q_len]
+
+
+def packed_mask_from_parents(parents: Sequence[int], device=None) -> torch.Tensor:
+    """[L, ceil(L/64)] packed ancestor-or-self mask of a parent array."""
+    m = pack_mask(ancestor_matrix(parents))
+    return m.to(device) if device is not None else m

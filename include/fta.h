@@ -39,6 +39,13 @@ typedef enum fta_status {
 
 typedef enum fta_dtype { FTA_F32 = 0, FTA_F16 = 1, FTA_BF16 = 2 } fta_dtype;
 typedef enum fta_len_dtype { FTA_I32 = 0, FTA_I64 = 1 } fta_len_dtype;
+/* Form of the tree mask. The reference adds a float tensor to the tree logits
+ * (flash_tree_attn.py:368); a draft tree only ever needs "attend / do not attend", which
+ * packs into one 64-bit word per query row and 64 tree positions. */
+typedef enum fta_mask_kind {
+  FTA_MASK_ADDITIVE_F32 = 0, /* float32, added to the tree logits (0 = attend, -inf = blocked, any other bias) */
+  FTA_MASK_PACKED_U64 = 1    /* uint64 [.., q_len, ceil(q_len/64)]: bit (j % 64) of word j / 64 set = row attends tree key j */
+} fta_mask_kind;
 
 /* Which stage-1 kernel a plan selects. */
 typedef enum fta_kernel {
@@ -54,7 +61,9 @@ typedef enum fta_kernel {
  *   k_cache   [bsz, num_kv_heads, cache_len, head_dim]   (same for v_cache)
  *   cur_k     [bsz, cur_heads, q_len, head_dim]          cur_heads = num_kv_heads or num_q_heads
  *   mask      float32, additive (flash_tree_attn.py:368); strides may be 0 to broadcast
- *             over batch and/or head, i.e. [q_len,q_len] .. [bsz,num_q_heads,q_len,q_len]
+ *             over batch and/or head, i.e. [q_len,q_len] .. [bsz,num_q_heads,q_len,q_len];
+ *             or, with mask_kind FTA_MASK_PACKED_U64, uint64 [.., q_len, ceil(q_len/64)]
+ *             (8 bytes per row and 64 tree keys instead of 256; strides in uint64 words)
  *   kv_seq_len[bsz] int32 or int64 (flash_tree_attn.py:434 passes int64)
  *   out       [bsz, num_q_heads, q_len, head_dim], dtype of q: the FINAL result
  *   mid_o     float32 [bsz, num_q_heads, mid_splits, q_len, head_dim]  (flash_tree_attn.py:276-279)
@@ -75,7 +84,7 @@ typedef struct fta_args {
   const void* v_cache;
   const void* cur_k;
   const void* cur_v;
-  const float* mask;
+  const void* mask;         /* float32 or uint64 words, see mask_kind */
   const void* kv_seq_len;
   void* out;
   float* mid_o;
@@ -98,6 +107,7 @@ typedef struct fta_args {
   int32_t force_splits;     /* 0 = heuristic; >0 pins the split count (tuning, tests) */
   int32_t force_kernel;     /* -1 = heuristic; else an fta_kernel */
   int32_t counter_elems;    /* int32 elements behind `counters`, 0 when it is NULL */
+  int32_t mask_kind;        /* fta_mask_kind of `mask` */
   float sm_scale;
 
   int64_t q_stride[3];      /* batch, head, row */
@@ -105,7 +115,7 @@ typedef struct fta_args {
   int64_t v_stride[3];
   int64_t ck_stride[3];     /* batch, head, row */
   int64_t cv_stride[3];
-  int64_t mask_stride[3];   /* batch, head, row (column stride is 1) */
+  int64_t mask_stride[3];   /* batch, head, row (column / word stride is 1), in elements of the mask's type */
   int64_t out_stride[3];    /* batch, head, row */
   int64_t mid_o_stride[4];  /* batch, head, split, row */
   int64_t mid_lse_stride[3];/* batch, head, split */

@@ -194,6 +194,30 @@ def test_mask_forms():
     check(run(x), oracle(x), torch.float16)
 
 
+@pytest.mark.parametrize("L,hq,hkv,D,dtype", [(64, 32, 8, 128, torch.bfloat16), (26, 4, 4, 128, torch.float16),
+                                              (130, 2, 1, 128, torch.float16), (5, 4, 2, 64, torch.float32),
+                                              (3, 8, 2, 128, torch.bfloat16)])
+def test_packed_mask_equals_additive_mask(L, hq, hkv, D, dtype):
+    """A 0 / -inf additive mask and its packed bit form (one uint64 word per row and 64
+    tree keys) must give identical results, in every broadcast form and in both kernels."""
+    from flash_tree_attn_amd.tree_mask import pack_mask
+    bsz = 3
+    x = make(71, bsz, hq, hkv, L, D, 300, dtype, [300, 17, 128])
+    g = torch.Generator().manual_seed(5)
+    allowed = (torch.rand(bsz, hq, L, L, generator=g) < 0.5) | torch.eye(L, dtype=torch.bool)
+    for view in (allowed[0, 0], allowed[:, :1], allowed):
+        add = torch.where(view, torch.zeros(()), torch.full((), -math.inf)).to(DEV)
+        xa, xp = dict(x, mask=add), dict(x, mask=pack_mask(view).to(DEV))
+        ref = oracle(xa)
+        out_add, out_packed = run(xa), run(xp)
+        check(out_packed, ref, dtype)
+        assert torch.equal(out_add, out_packed)
+        if dtype != torch.float32:
+            assert torch.equal(run(xa, _force_kernel=_lib.KERNEL_SHUFFLE), run(xp, _force_kernel=_lib.KERNEL_SHUFFLE))
+    with pytest.raises(ValueError):
+        run(dict(x, mask=torch.zeros(L, (L + 63) // 64 + 1, dtype=torch.int64, device=DEV)))
+
+
 def test_fully_masked_rows_and_empty_cache():
     x = make(17, 2, 4, 2, 20, 128, 64, torch.bfloat16, [0, 40])
     x["mask"] = x["mask"].clone()
