@@ -15,7 +15,7 @@ KERNEL_SHUFFLE, KERNEL_MFMA = 0, 1
 
 EXPORTED_SYMBOLS = (
     "fta_abi_version", "fta_strerror", "fta_validate", "fta_plan", "fta_decode", "fta_decode_stage1",
-    "fta_decode_stage2", "fta_device_cus",
+    "fta_decode_stage2", "fta_device_cus", "fta_append_kv",
 )
 
 # status -> Python exception class
@@ -36,6 +36,17 @@ class FtaArgs(C.Structure):
         ("q_stride", C.c_int64 * 3), ("k_stride", C.c_int64 * 3), ("v_stride", C.c_int64 * 3),
         ("ck_stride", C.c_int64 * 3), ("cv_stride", C.c_int64 * 3), ("mask_stride", C.c_int64 * 3),
         ("out_stride", C.c_int64 * 3), ("mid_o_stride", C.c_int64 * 4), ("mid_lse_stride", C.c_int64 * 3),
+    ]
+
+
+class FtaAppendArgs(C.Structure):
+    _fields_ = [
+        ("k_cache", C.c_void_p), ("v_cache", C.c_void_p), ("cur_k", C.c_void_p), ("cur_v", C.c_void_p),
+        ("accept_idx", C.c_void_p), ("accept_len", C.c_void_p), ("kv_seq_len", C.c_void_p), ("kv_seq_len_out", C.c_void_p),
+        ("bsz", C.c_int32), ("num_kv_heads", C.c_int32), ("q_len", C.c_int32), ("head_dim", C.c_int32),
+        ("cache_len", C.c_int32), ("max_accept", C.c_int32), ("dtype", C.c_int32), ("len_dtype", C.c_int32),
+        ("k_stride", C.c_int64 * 3), ("v_stride", C.c_int64 * 3), ("ck_stride", C.c_int64 * 3), ("cv_stride", C.c_int64 * 3),
+        ("accept_idx_stride", C.c_int64),
     ]
 
 
@@ -82,6 +93,8 @@ def load() -> C.CDLL:
         fn.restype = C.c_int
         fn.argtypes = [C.POINTER(FtaArgs), C.c_void_p]
     lib.fta_device_cus.restype = C.c_int
+    lib.fta_append_kv.restype = C.c_int
+    lib.fta_append_kv.argtypes = [C.POINTER(FtaAppendArgs), C.c_void_p]
     if lib.fta_abi_version() != ABI_VERSION:
         raise ImportError(f"libfta.so has ABI {lib.fta_abi_version()}, binding expects {ABI_VERSION}; rebuild it")
     _lib = lib

@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 LIB_PATH = os.path.join(HERE, "libfta.so")
-SOURCES = ["fta_host.cpp", "stage1_shuffle.hip", "stage1_mfma.hip", "stage2_merge.hip"]
+SOURCES = ["fta_host.cpp", "stage1_shuffle.hip", "stage1_mfma.hip", "stage2_merge.hip", "append_kv.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
@@ -43,7 +43,7 @@ def _compile(src: str) -> str:
 
 
 def build(verbose: bool = True) -> str:
-    with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as pool:
+    with ThreadPoolExecutor(max_workers=min(5, len(SOURCES))) as pool:
         objs = list(pool.map(_compile, SOURCES))
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", *objs, "-o", LIB_PATH]
     res = subprocess.run(cmd, capture_output=True, text=True)

@@ -1,0 +1,83 @@
+"""`append_accepted_kv`: writes the accepted path of the draft tree into the KV cache.
+
+The step that follows `flash_decoding_attention` in a speculative-decoding loop; the
+reference leaves it to its caller (README.md:63-64). Runs a gfx950 copy kernel through
+the C ABI (`fta_append_kv`, include/fta.h); GPU tensors only, no fallback.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional
+
+import torch
+
+from . import _lib
+from .flash_decoding import _DTYPES, _check, _rows_ok
+
+
+def append_accepted_kv(k_cache: torch.Tensor, v_cache: torch.Tensor, current_k: torch.Tensor, current_v: torch.Tensor,
+                       accept_idx: torch.Tensor, accept_len: torch.Tensor, kv_seq_len: torch.Tensor,
+                       out_kv_seq_len: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """For every sequence b and a < accept_len[b]:
+        k_cache[b, :, kv_seq_len[b] + a] = current_k[b, :, accept_idx[b, a]]   (same for v)
+    and the returned lengths are kv_seq_len + accept_len (clamped to the cache capacity;
+    rows past it are dropped). `k_cache` / `v_cache` are updated in place; the lengths go
+    to `out_kv_seq_len`, or in place into `kv_seq_len` when it is None.
+
+      k_cache / v_cache   [bsz, num_kv_heads, cache_len, head_dim]
+      current_k / _v      [bsz, num_kv_heads, q_len, head_dim]
+      accept_idx          int32 [bsz, max_accept]: tree positions of the accepted path, root first
+      accept_len          [bsz], dtype of kv_seq_len (int32 or int64)
+    """
+    lib = _lib.load()
+    dev = k_cache.device
+    if dev.type != "cuda":
+        raise RuntimeError("append_accepted_kv runs on the GPU only; there is no CPU fallback")
+    if k_cache.dim() != 4 or k_cache.shape != v_cache.shape:
+        raise ValueError("k_cache / v_cache must be [bsz, num_kv_heads, cache_len, head_dim] and alike")
+    bsz, hkv, cache_len, D = k_cache.shape
+    if k_cache.dtype not in _DTYPES:
+        raise ValueError(f"unsupported dtype {k_cache.dtype}")
+    if current_k.shape != current_v.shape or current_k.dim() != 4 or current_k.size(0) != bsz or current_k.size(3) != D:
+        raise ValueError("current_k / current_v must be [bsz, num_kv_heads, q_len, head_dim]")
+    if current_k.size(1) != hkv:
+        raise ValueError("only tree K/V with num_kv_heads heads can be appended to the cache")
+    for t in (v_cache, current_k, current_v):
+        if t.dtype != k_cache.dtype or t.device != dev:
+            raise ValueError("caches and tree K/V must share dtype and device")
+    for name, t in (("k_cache", k_cache), ("v_cache", v_cache)):
+        if not _rows_ok(t):
+            raise ValueError(f"{name} needs unit inner stride and 16-byte aligned rows (it is updated in place)")
+    current_k = current_k if _rows_ok(current_k) else current_k.contiguous()
+    current_v = current_v if _rows_ok(current_v) else current_v.contiguous()
+    if accept_idx.dim() != 2 or accept_idx.size(0) != bsz or accept_idx.dtype != torch.int32 or accept_idx.device != dev:
+        raise ValueError("accept_idx must be an int32 tensor [bsz, max_accept] on the caches' device")
+    if accept_idx.stride(1) != 1 and accept_idx.size(1) > 1:
+        accept_idx = accept_idx.contiguous()
+    if kv_seq_len.dtype not in (torch.int32, torch.int64) or kv_seq_len.numel() != bsz or kv_seq_len.device != dev:
+        raise ValueError("kv_seq_len must be an int32/int64 tensor of bsz elements on the caches' device")
+    if accept_len.dtype != kv_seq_len.dtype or accept_len.numel() != bsz or accept_len.device != dev:
+        raise ValueError("accept_len must match kv_seq_len in dtype, size and device")
+    if not kv_seq_len.is_contiguous():
+        raise ValueError("kv_seq_len must be contiguous (it is updated in place)")
+    accept_len = accept_len.contiguous().view(-1)
+    out = kv_seq_len if out_kv_seq_len is None else out_kv_seq_len
+    if out.dtype != kv_seq_len.dtype or out.numel() != bsz or out.device != dev or not out.is_contiguous():
+        raise ValueError("out_kv_seq_len must match kv_seq_len in dtype, size and device, and be contiguous")
+
+    a = _lib.FtaAppendArgs()
+    a.k_cache, a.v_cache, a.cur_k, a.cur_v = k_cache.data_ptr(), v_cache.data_ptr(), current_k.data_ptr(), current_v.data_ptr()
+    a.accept_idx, a.accept_len = accept_idx.data_ptr(), accept_len.data_ptr()
+    a.kv_seq_len, a.kv_seq_len_out = kv_seq_len.data_ptr(), out.data_ptr()
+    a.bsz, a.num_kv_heads, a.q_len, a.head_dim = bsz, hkv, current_k.size(2), D
+    a.cache_len, a.max_accept = cache_len, accept_idx.size(1)
+    a.dtype = _DTYPES[k_cache.dtype]
+    a.len_dtype = _lib.FTA_I64 if kv_seq_len.dtype == torch.int64 else _lib.FTA_I32
+    a.k_stride[:] = k_cache.stride()[:3]
+    a.v_stride[:] = v_cache.stride()[:3]
+    a.ck_stride[:] = current_k.stride()[:3]
+    a.cv_stride[:] = current_v.stride()[:3]
+    a.accept_idx_stride = accept_idx.stride(0)
+    with torch.cuda.device(dev):
+        _check(lib.fta_append_kv(C.byref(a), C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)))
+    return out

@@ -171,6 +171,48 @@ int fta_decode(const fta_args* args, void* hip_stream);
 int fta_decode_stage1(const fta_args* args, void* hip_stream);
 int fta_decode_stage2(const fta_args* args, void* hip_stream);
 
+/*
+ * Accepted-path KV append: the step that follows this op in a speculative-decoding loop
+ * (the reference leaves it to the caller: README.md:63-64 "kv cache management"). For
+ * every sequence b and a < accept_len[b]:
+ *     k_cache[b, h, T_b + a, :] = cur_k[b, h, accept_idx[b, a], :]      (same for v)
+ * with T_b = kv_seq_len[b], then kv_seq_len_out[b] = T_b + accept_len[b]. Rows that would
+ * land past cache_len are dropped and the new length is clamped to cache_len (there is
+ * no host sync to report it). accept_len is clamped to [0, max_accept]; an accept_idx
+ * outside [0, q_len) drops that row's copy but still counts it. Strides in elements,
+ * inner stride 1, rows 16-byte aligned, as for fta_args. kv_seq_len_out may alias
+ * kv_seq_len (in-place update; then the lengths are written by a second, one-block
+ * launch after the copies have read them).
+ */
+typedef struct fta_append_args {
+  void* k_cache;             /* [bsz, num_kv_heads, cache_len, head_dim] */
+  void* v_cache;
+  const void* cur_k;         /* [bsz, num_kv_heads, q_len, head_dim] */
+  const void* cur_v;
+  const int32_t* accept_idx; /* [bsz, max_accept] tree positions of the accepted path, in order */
+  const void* accept_len;    /* [bsz], len_dtype */
+  const void* kv_seq_len;    /* [bsz], len_dtype */
+  void* kv_seq_len_out;      /* [bsz], len_dtype */
+
+  int32_t bsz;
+  int32_t num_kv_heads;
+  int32_t q_len;
+  int32_t head_dim;
+  int32_t cache_len;
+  int32_t max_accept;
+  int32_t dtype;             /* fta_dtype */
+  int32_t len_dtype;         /* fta_len_dtype of accept_len, kv_seq_len and kv_seq_len_out */
+
+  int64_t k_stride[3];       /* batch, head, position */
+  int64_t v_stride[3];
+  int64_t ck_stride[3];      /* batch, head, row */
+  int64_t cv_stride[3];
+  int64_t accept_idx_stride; /* batch stride of accept_idx */
+} fta_append_args;
+
+/* Validates, then launches on `hip_stream`. Asynchronous; allocates nothing. */
+int fta_append_kv(const fta_append_args* args, void* hip_stream);
+
 /* Number of compute units of the current HIP device, or a negative fta_status. */
 int fta_device_cus(void);
 

@@ -58,20 +58,24 @@ def test_struct_layout_matches_header(fta_lib, tmp_path):
     # ... and field by field against what a C compiler makes of include/fta.h
     fields = [n for n, _ in _lib.FtaArgs._fields_]
     plan_fields = [n for n, _ in _lib.FtaPlanOut._fields_]
+    append_fields = [n for n, _ in _lib.FtaAppendArgs._fields_]
     src = tmp_path / "layout.c"
     lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "fta.h"', 'int main(void) {',
-             '  printf("%zu %zu\\n", sizeof(fta_args), sizeof(fta_plan_out));']
+             '  printf("%zu %zu %zu\\n", sizeof(fta_args), sizeof(fta_plan_out), sizeof(fta_append_args));']
     lines += [f'  printf("%zu\\n", offsetof(fta_args, {n}));' for n in fields]
     lines += [f'  printf("%zu\\n", offsetof(fta_plan_out, {n}));' for n in plan_fields]
+    lines += [f'  printf("%zu\\n", offsetof(fta_append_args, {n}));' for n in append_fields]
     lines += ['  return 0;', '}']
     src.write_text("\n".join(lines))
     exe = tmp_path / "layout"
     subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
     out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
-    assert [int(out[0]), int(out[1])] == [C.sizeof(_lib.FtaArgs), C.sizeof(_lib.FtaPlanOut)]
-    offs = [int(v) for v in out[2:]]
-    assert offs[:len(fields)] == [getattr(_lib.FtaArgs, n).offset for n in fields]
-    assert offs[len(fields):] == [getattr(_lib.FtaPlanOut, n).offset for n in plan_fields]
+    assert [int(v) for v in out[:3]] == [C.sizeof(_lib.FtaArgs), C.sizeof(_lib.FtaPlanOut), C.sizeof(_lib.FtaAppendArgs)]
+    offs = [int(v) for v in out[3:]]
+    n1, n2 = len(fields), len(fields) + len(plan_fields)
+    assert offs[:n1] == [getattr(_lib.FtaArgs, n).offset for n in fields]
+    assert offs[n1:n2] == [getattr(_lib.FtaPlanOut, n).offset for n in plan_fields]
+    assert offs[n2:] == [getattr(_lib.FtaAppendArgs, n).offset for n in append_fields]
 
 
 def test_strerror(fta_lib):

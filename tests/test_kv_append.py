@@ -1,0 +1,179 @@
+"""Accepted-path KV append (`fta_append_kv`, include/fta.h): the oracle against torch's
+own indexing on CPU, argument errors of the C entry point without a GPU, and bit-exact
+GPU parity (it is a copy: no tolerance)."""
+import ctypes as C
+
+import pytest
+import torch
+
+from flash_tree_attn_amd import _lib
+from oracle.kv_append_oracle import append_accepted_kv_oracle
+
+DEV = "cuda"
+
+
+def make(seed, bsz, hkv, L, D, cache_len, dtype, lens, acc, max_accept, len_dtype=torch.int64):
+    g = torch.Generator().manual_seed(seed)
+    r = lambda *s: torch.randn(*s, generator=g).to(dtype)
+    x = dict(k_cache=r(bsz, hkv, cache_len, D), v_cache=r(bsz, hkv, cache_len, D), current_k=r(bsz, hkv, L, D),
+             current_v=r(bsz, hkv, L, D))
+    idx = torch.stack([torch.randperm(L, generator=g)[:max_accept] if L >= max_accept
+                       else torch.randint(0, L, (max_accept,), generator=g) for _ in range(bsz)]).to(torch.int32)
+    x["accept_idx"] = idx
+    x["accept_len"] = torch.tensor(acc, dtype=len_dtype)
+    x["kv_seq_len"] = torch.tensor(lens, dtype=len_dtype)
+    return x
+
+
+# ---------------------------------------------------------------- CPU
+def test_oracle_equals_torch_indexing():
+    x = make(1, 3, 2, 10, 8, 40, torch.float32, [5, 38, 0], [4, 4, 0], 4)
+    k, v, n = append_accepted_kv_oracle(**x)
+    for b, (t, a) in enumerate(zip([5, 38, 0], [4, 4, 0])):
+        room = min(a, 40 - t)
+        sel = x["accept_idx"][b, :room].long()
+        exp_k = x["k_cache"][b].clone()
+        exp_k[:, t:t + room] = x["current_k"][b].index_select(1, sel)
+        exp_v = x["v_cache"][b].clone()
+        exp_v[:, t:t + room] = x["current_v"][b].index_select(1, sel)
+        assert torch.equal(k[b], exp_k) and torch.equal(v[b], exp_v)
+    assert n.tolist() == [9, 40, 0]
+
+
+def base_args(**kw):
+    a = _lib.FtaAppendArgs()
+    for f in ("k_cache", "v_cache", "cur_k", "cur_v", "accept_idx", "accept_len", "kv_seq_len", "kv_seq_len_out"):
+        setattr(a, f, 0x1000)
+    cfg = dict(bsz=2, num_kv_heads=4, q_len=8, head_dim=128, cache_len=64, max_accept=4, dtype=_lib.FTA_BF16,
+               len_dtype=_lib.FTA_I64)
+    cfg.update(kw)
+    for k, v in cfg.items():
+        setattr(a, k, v)
+    D, L, T, H = a.head_dim, a.q_len, a.cache_len, a.num_kv_heads
+    a.k_stride[:] = [H * T * D, T * D, D]
+    a.v_stride[:] = a.k_stride[:]
+    a.ck_stride[:] = [H * L * D, L * D, D]
+    a.cv_stride[:] = a.ck_stride[:]
+    a.accept_idx_stride = a.max_accept
+    return a
+
+
+def test_append_argument_errors_without_touching_the_gpu(fta_lib):
+    assert fta_lib.fta_append_kv(None, None) == -1
+    a = base_args()
+    a.accept_idx = None
+    assert fta_lib.fta_append_kv(C.byref(a), None) == -1
+    assert fta_lib.fta_append_kv(C.byref(base_args(head_dim=100)), None) == -2
+    assert fta_lib.fta_append_kv(C.byref(base_args(dtype=9)), None) == -6
+    assert fta_lib.fta_append_kv(C.byref(base_args(bsz=0)), None) == -7
+    a = base_args()
+    a.k_stride[2] = 100
+    assert fta_lib.fta_append_kv(C.byref(a), None) == -8
+    a = base_args()
+    a.cur_v = 0x1008
+    assert fta_lib.fta_append_kv(C.byref(a), None) == -8
+    if not torch.cuda.is_available():
+        assert fta_lib.fta_append_kv(C.byref(base_args()), None) == -11
+
+
+def test_python_wrapper_rejects_cpu_tensors():
+    from flash_tree_attn_amd import append_accepted_kv
+    x = make(2, 1, 1, 4, 32, 8, torch.float16, [2], [1], 2)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        append_accepted_kv(**x)
+
+
+# ---------------------------------------------------------------- GPU
+def gpu_run(x, out_of_place=False):
+    from flash_tree_attn_amd import append_accepted_kv
+    d = {k: v.to(DEV) for k, v in x.items()}
+    out = torch.full_like(d["kv_seq_len"], -7) if out_of_place else None
+    old = d["kv_seq_len"].clone()
+    ret = append_accepted_kv(**d, out_kv_seq_len=out)
+    if out_of_place:
+        assert torch.equal(d["kv_seq_len"], old) and ret is out
+    else:
+        assert ret is d["kv_seq_len"]
+    return d["k_cache"].cpu(), d["v_cache"].cpu(), ret.cpu()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("out_of_place", [False, True])
+def test_append_matches_oracle_bit_for_bit(dtype, out_of_place):
+    # ragged accept lengths incl. 0, a sequence that hits the cache capacity, an empty cache
+    x = make(3, 5, 3, 16, 128, 96, dtype, [10, 93, 0, 96, 50], [6, 6, 1, 3, 0], 6)
+    k, v, n = append_accepted_kv_oracle(**x)
+    gk, gv, gn = gpu_run(x, out_of_place)
+    assert torch.equal(gk, k) and torch.equal(gv, v) and torch.equal(gn, n)
+    assert n.tolist() == [16, 96, 1, 96, 50]
+
+
+@pytest.mark.gpu
+def test_append_edge_cases():
+    # int32 lengths, head_dim 32 and 256, out-of-range tree positions are dropped but counted,
+    # accept_len beyond max_accept and negative lengths are clamped
+    for D in (32, 256):
+        x = make(4, 3, 2, 5, D, 20, torch.float16, [3, 7, -2], [9, 2, 3], 4, len_dtype=torch.int32)
+        x["accept_idx"][1, 0] = 5
+        x["accept_idx"][1, 1] = -1
+        k, v, n = append_accepted_kv_oracle(**x)
+        gk, gv, gn = gpu_run(x)
+        assert torch.equal(gk, k) and torch.equal(gv, v) and torch.equal(gn, n)
+        assert n.tolist() == [7, 9, 3] and gn.dtype == torch.int32
+        assert torch.equal(gk[1], x["k_cache"][1])   # nothing valid to copy for sequence 1
+
+
+@pytest.mark.gpu
+def test_append_into_strided_cache_views():
+    from flash_tree_attn_amd import append_accepted_kv
+    x = make(5, 2, 2, 8, 64, 32, torch.bfloat16, [4, 30], [3, 3], 3)
+    kv = torch.zeros(2, 2, 2, 32, 64, dtype=torch.bfloat16)   # [bsz, K|V, heads, T, D], as the reference benchmark slices
+    kv[:, 0], kv[:, 1] = x["k_cache"], x["v_cache"]
+    d = {k: v.to(DEV) for k, v in x.items()}
+    kvd = kv.to(DEV)
+    d["k_cache"], d["v_cache"] = kvd[:, 0], kvd[:, 1]
+    append_accepted_kv(**d)
+    k, v, n = append_accepted_kv_oracle(**x)
+    assert torch.equal(kvd[:, 0].cpu(), k) and torch.equal(kvd[:, 1].cpu(), v) and torch.equal(d["kv_seq_len"].cpu(), n)
+
+
+@pytest.mark.gpu
+def test_speculative_loop_decode_append_decode():
+    """Two verification steps with an append in between equal the oracle run on a cache
+    that was extended by hand."""
+    from flash_tree_attn_amd import append_accepted_kv, flash_decoding_attention
+    from flash_tree_attn_amd.tree_mask import additive_mask_from_parents, random_tree_parents
+    from oracle.tree_attn_oracle import tree_attention_oracle
+    g = torch.Generator().manual_seed(9)
+    bsz, hq, hkv, L, D, cap = 2, 8, 2, 12, 128, 256
+    r = lambda *s: torch.randn(*s, generator=g).to(torch.bfloat16).to(DEV)
+    k_cache, v_cache = r(bsz, hkv, cap, D), r(bsz, hkv, cap, D)
+    lens = torch.tensor([100, 37], dtype=torch.int64, device=DEV)
+    ref_k, ref_v, ref_lens = k_cache.clone(), v_cache.clone(), lens.clone()
+    for step in range(2):
+        parents = random_tree_parents(L, g)
+        mask = additive_mask_from_parents(parents, device=DEV)
+        q, ck, cv = r(bsz, hq, L, D), r(bsz, hkv, L, D), r(bsz, hkv, L, D)
+        out = flash_decoding_attention(q, k_cache, v_cache, ck, cv, mask, lens, kv_group_num=hq // hkv)
+        ref = tree_attention_oracle(q, ref_k, ref_v, ck, cv, mask, ref_lens, None, hq // hkv)
+        torch.testing.assert_close(out.float(), ref, atol=2e-3, rtol=1e-2)
+        # accept a root-to-node path: walk up from a random node
+        paths = []
+        for b in range(bsz):
+            node, path = int(torch.randint(0, L, (1,), generator=g)), []
+            while node >= 0:
+                path.append(node)
+                node = int(parents[node])
+            paths.append(path[::-1])
+        n_acc = torch.tensor([len(p) for p in paths], dtype=torch.int64, device=DEV)
+        idx = torch.zeros(bsz, L, dtype=torch.int32)
+        for b, pth in enumerate(paths):
+            idx[b, :len(pth)] = torch.tensor(pth, dtype=torch.int32)
+        append_accepted_kv(k_cache, v_cache, ck, cv, idx.to(DEV), n_acc, lens)
+        for b, pth in enumerate(paths):
+            t = int(ref_lens[b])
+            ref_k[b, :, t:t + len(pth)] = ck[b][:, pth]
+            ref_v[b, :, t:t + len(pth)] = cv[b][:, pth]
+            ref_lens[b] = t + len(pth)
+        assert torch.equal(lens, ref_lens) and torch.equal(k_cache, ref_k) and torch.equal(v_cache, ref_v)
