@@ -30,6 +30,8 @@ def parse():
     ap.add_argument("--config", default="cfg3_gqa_8b_bf16", help="workload name (flash_tree_attn_amd.synthetic.CONFIGS)")
     ap.add_argument("--kv-sets", type=int, default=0, help="independent KV caches to rotate over (0 = enough for >1 GiB)")
     ap.add_argument("--splits", type=int, default=0, help="pin the split count (0 = heuristic)")
+    ap.add_argument("--paged", type=int, default=0, metavar="PAGE",
+                    help="run on paged caches: pages of PAGE positions (16/32/64/128), shuffled in one pool, with a block table")
     ap.add_argument("--packed-mask", action="store_true", help="pass the tree mask as packed bit words instead of float32")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -122,9 +124,29 @@ def main():
     if args.packed_mask:
         from flash_tree_attn_amd.tree_mask import pack_mask
         mask_arg = pack_mask(x["mask"])
-    calls = [prepare(x["q"], kc, vc, x["current_k"], x["current_v"], mask_arg, x["kv_seq_len"], cfg.block_size,
-                     None, None, None, None, x["sm_scale"], cfg.kv_group_num, _force_splits=args.splits)
-             for kc, vc in zip(x["k_caches"], x["v_caches"])]
+    def paged(kc, vc, seed):
+        """The same cache as a pool of shuffled pages plus its block table."""
+        bsz, hkv, t, d = kc.shape
+        pg, per_seq = args.paged, kc.shape[2] // args.paged
+        perm = torch.randperm(bsz * per_seq, generator=torch.Generator().manual_seed(seed)).to(dev)
+        pool = lambda c: c.view(bsz, hkv, per_seq, pg, d).permute(0, 2, 1, 3, 4).reshape(bsz * per_seq, hkv, pg, d)
+        kp, vp = torch.empty_like(pool(kc)), torch.empty_like(pool(vc))
+        kp[perm], vp[perm] = pool(kc), pool(vc)
+        return kp, vp, perm.view(bsz, per_seq).to(torch.int32)
+
+    calls = []
+    for i, (kc, vc) in enumerate(zip(x["k_caches"], x["v_caches"])):
+        tables = None
+        if args.paged:
+            assert cfg.cache_len % args.paged == 0
+            kc, vc, tables = paged(kc, vc, i)
+            if i == 0:
+                x["k_cache_paged"], x["v_cache_paged"], x["tables"] = kc, vc, tables
+        calls.append(prepare(x["q"], kc, vc, x["current_k"], x["current_v"], mask_arg, x["kv_seq_len"], cfg.block_size,
+                             None, None, None, None, x["sm_scale"], cfg.kv_group_num, _force_splits=args.splits,
+                             block_tables=tables))
+    if args.paged:   # the contiguous copies are no longer needed, except set 0 for the self-check
+        x["k_caches"], x["v_caches"] = x["k_caches"][:1], x["v_caches"][:1]
     plan = calls[0].plan
     nbytes = algorithmic_bytes(cfg, x["kv_seq_len"].cpu(), mask_arg)
     nflops = flops(cfg, x["kv_seq_len"].cpu())
@@ -170,7 +192,8 @@ def main():
         "data": "synthetic (seed 0, N(0,1) q/k/v, random tree mask), inputs resident in HBM",
         "config": {"workload": cfg.name, "bsz": cfg.bsz, "q_heads": cfg.num_heads, "kv_heads": cfg.num_kv_heads,
                    "head_dim": cfg.head_dim, "q_len": cfg.q_len, "cache_len": cfg.cache_len, "lengths": cfg.lengths,
-                   "block_size": cfg.block_size, "mask": "packed u64" if args.packed_mask else "additive f32", "kv_sets_rotated": kv_sets, "num_splits": plan.num_splits,
+                   "block_size": cfg.block_size, "mask": "packed u64" if args.packed_mask else "additive f32",
+                   "kv_layout": f"paged, {args.paged} positions per page, shuffled pool" if args.paged else "contiguous per sequence", "kv_sets_rotated": kv_sets, "num_splits": plan.num_splits,
                    "chunk": plan.chunk, "stage1_kernel": "mfma" if plan.kernel == _lib.KERNEL_MFMA else "shuffle",
                    "stage1_workgroups": plan.num_workgroups, "algorithmic_bytes": nbytes, "flops": nflops},
         "tflops": nflops / (ms * 1e-3) / 1e12,

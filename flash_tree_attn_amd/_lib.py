@@ -27,15 +27,16 @@ class FtaArgs(C.Structure):
         ("q", C.c_void_p), ("k_cache", C.c_void_p), ("v_cache", C.c_void_p),
         ("cur_k", C.c_void_p), ("cur_v", C.c_void_p), ("mask", C.c_void_p),
         ("kv_seq_len", C.c_void_p), ("out", C.c_void_p), ("mid_o", C.c_void_p), ("mid_lse", C.c_void_p),
-        ("counters", C.c_void_p),
+        ("counters", C.c_void_p), ("block_table", C.c_void_p),
         ("bsz", C.c_int32), ("num_q_heads", C.c_int32), ("num_kv_heads", C.c_int32), ("cur_heads", C.c_int32),
         ("q_len", C.c_int32), ("head_dim", C.c_int32), ("cache_len", C.c_int32), ("v_cache_len", C.c_int32),
         ("block_size", C.c_int32), ("max_seq_len_hint", C.c_int32), ("mid_splits", C.c_int32),
         ("dtype", C.c_int32), ("len_dtype", C.c_int32), ("force_splits", C.c_int32), ("force_kernel", C.c_int32),
-        ("counter_elems", C.c_int32), ("mask_kind", C.c_int32), ("sm_scale", C.c_float),
+        ("counter_elems", C.c_int32), ("mask_kind", C.c_int32), ("page_size", C.c_int32), ("sm_scale", C.c_float),
         ("q_stride", C.c_int64 * 3), ("k_stride", C.c_int64 * 3), ("v_stride", C.c_int64 * 3),
         ("ck_stride", C.c_int64 * 3), ("cv_stride", C.c_int64 * 3), ("mask_stride", C.c_int64 * 3),
         ("out_stride", C.c_int64 * 3), ("mid_o_stride", C.c_int64 * 4), ("mid_lse_stride", C.c_int64 * 3),
+        ("block_table_stride", C.c_int64),
     ]
 
 
@@ -43,10 +44,12 @@ class FtaAppendArgs(C.Structure):
     _fields_ = [
         ("k_cache", C.c_void_p), ("v_cache", C.c_void_p), ("cur_k", C.c_void_p), ("cur_v", C.c_void_p),
         ("accept_idx", C.c_void_p), ("accept_len", C.c_void_p), ("kv_seq_len", C.c_void_p), ("kv_seq_len_out", C.c_void_p),
+        ("block_table", C.c_void_p),
         ("bsz", C.c_int32), ("num_kv_heads", C.c_int32), ("q_len", C.c_int32), ("head_dim", C.c_int32),
         ("cache_len", C.c_int32), ("max_accept", C.c_int32), ("dtype", C.c_int32), ("len_dtype", C.c_int32),
+        ("page_size", C.c_int32), ("reserved", C.c_int32),
         ("k_stride", C.c_int64 * 3), ("v_stride", C.c_int64 * 3), ("ck_stride", C.c_int64 * 3), ("cv_stride", C.c_int64 * 3),
-        ("accept_idx_stride", C.c_int64),
+        ("accept_idx_stride", C.c_int64), ("block_table_stride", C.c_int64),
     ]
 
 

@@ -20,12 +20,14 @@ struct AppendParams {
   char* k; char* v;
   const char* ck; const char* cv;
   const int32_t* idx;
+  const int32_t* table;  // null = contiguous caches
   const void* acc_len; const void* lens; void* lens_out;
   int32_t bsz, heads, q_len, cache_len, max_accept, len_is_i64;
   int32_t row_bytes;     // head_dim * element size
   int32_t write_lens;    // 1: this launch also writes the new lengths (out does not alias in)
   int64_t k_stride[3], v_stride[3], ck_stride[3], cv_stride[3];   // in BYTES
-  int64_t idx_stride;
+  int64_t idx_stride, table_stride;
+  int32_t page_shift;
 };
 
 __device__ __forceinline__ int clamp_i64(int64_t v, int lo, int hi) {
@@ -61,8 +63,13 @@ __global__ void __launch_bounds__(256) append_kv_kernel(const AppendParams p) {
   if (src_row < 0 || src_row >= p.q_len) return;
   const char* src = is_v ? p.cv + b * p.cv_stride[0] + h * p.cv_stride[1] + src_row * p.cv_stride[2]
                          : p.ck + b * p.ck_stride[0] + h * p.ck_stride[1] + src_row * p.ck_stride[2];
-  char* dst = is_v ? p.v + b * p.v_stride[0] + h * p.v_stride[1] + static_cast<int64_t>(t + a) * p.v_stride[2]
-                   : p.k + b * p.k_stride[0] + h * p.k_stride[1] + static_cast<int64_t>(t + a) * p.k_stride[2];
+  int64_t outer = b, pos = t + a;   // contiguous: [batch, head, position]
+  if (p.table) {                     // paged: [page, head, position in page]
+    outer = p.table[b * p.table_stride + (pos >> p.page_shift)];
+    pos &= (1 << p.page_shift) - 1;
+  }
+  char* dst = is_v ? p.v + outer * p.v_stride[0] + h * p.v_stride[1] + pos * p.v_stride[2]
+                   : p.k + outer * p.k_stride[0] + h * p.k_stride[1] + pos * p.k_stride[2];
   *reinterpret_cast<u32x4*>(dst + piece * 16) = *reinterpret_cast<const u32x4*>(src + piece * 16);
 }
 
@@ -89,6 +96,10 @@ extern "C" int fta_append_kv(const fta_append_args* args, void* hip_stream) {
   if (a.head_dim != 32 && a.head_dim != 64 && a.head_dim != 128 && a.head_dim != 256) return FTA_ERR_HEAD_DIM;
   if (a.bsz <= 0 || a.num_kv_heads <= 0 || a.q_len <= 0 || a.cache_len < 0 || a.max_accept < 0 || a.accept_idx_stride < 0)
     return FTA_ERR_SHAPE;
+  if (a.block_table) {
+    if (a.page_size != 16 && a.page_size != 32 && a.page_size != 64 && a.page_size != 128) return FTA_ERR_BLOCK_SIZE;
+    if (a.block_table_stride < 0 || a.block_table_stride * a.page_size < a.cache_len) return FTA_ERR_SHAPE;
+  }
   const int es = a.dtype == FTA_F32 ? 4 : 2;
   const int vec = 16 / es;
   const int64_t* strides[] = {a.k_stride, a.v_stride, a.ck_stride, a.cv_stride};
@@ -113,6 +124,8 @@ extern "C" int fta_append_kv(const fta_append_args* args, void* hip_stream) {
     p.ck_stride[i] = a.ck_stride[i] * es; p.cv_stride[i] = a.cv_stride[i] * es;
   }
   p.idx_stride = a.accept_idx_stride;
+  p.table = a.block_table; p.table_stride = a.block_table_stride;
+  p.page_shift = a.page_size == 16 ? 4 : a.page_size == 32 ? 5 : a.page_size == 64 ? 6 : 7;
 
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return FTA_ERR_NO_DEVICE;

@@ -42,6 +42,17 @@ __device__ __forceinline__ float tree_mask_value(const KernelParams& p, int64_t 
   return static_cast<const float*>(p.mask)[row_start + j];
 }
 
+// Element offset of cache position `pos` of sequence b inside the K (or V) tensor, head
+// term excluded: batch stride x b for contiguous caches, page stride x page for paged
+// ones (stride[0] is the page stride then).
+__device__ __forceinline__ int64_t cache_row_offset(const KernelParams& p, const int64_t (&stride)[3], int b, int pos) {
+  if (p.block_table) {
+    const int page = p.block_table[b * p.table_stride + (pos >> p.page_shift)];
+    return page * stride[0] + (pos & ((1 << p.page_shift) - 1)) * stride[2];
+  }
+  return b * stride[0] + pos * stride[2];
+}
+
 // Splits that hold data for a sequence of `t` cached keys: ceil(t / chunk), at
 // least one (the tree block always needs a home), at most the grid extent.
 __device__ __forceinline__ int splits_for(int t, int chunk, int num_splits) {

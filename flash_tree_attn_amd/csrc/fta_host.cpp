@@ -45,6 +45,10 @@ int validate(const fta_args& a) {
   if (a.dtype != FTA_F32 && a.dtype != FTA_F16 && a.dtype != FTA_BF16) return FTA_ERR_DTYPE;
   if (a.len_dtype != FTA_I32 && a.len_dtype != FTA_I64) return FTA_ERR_DTYPE;
   if (a.mask_kind != FTA_MASK_ADDITIVE_F32 && a.mask_kind != FTA_MASK_PACKED_U64) return FTA_ERR_DTYPE;
+  if (a.block_table) {
+    if (a.page_size != 16 && a.page_size != 32 && a.page_size != 64 && a.page_size != 128) return FTA_ERR_BLOCK_SIZE;
+    if (a.block_table_stride < 0 || a.block_table_stride * a.page_size < a.cache_len) return FTA_ERR_SHAPE;
+  }
   if (a.head_dim != 32 && a.head_dim != 64 && a.head_dim != 128 && a.head_dim != 256) return FTA_ERR_HEAD_DIM;
   if (a.cache_len != a.v_cache_len) return FTA_ERR_CACHE_LEN_MISMATCH;
   if (a.block_size != 16 && a.block_size != 32 && a.block_size != 64 && a.block_size != 128)
@@ -247,6 +251,9 @@ int decode_impl(const fta_args* args, void* hip_stream, int stages) {
   p.q = a.q; p.k = a.k_cache; p.v = a.v_cache; p.ck = a.cur_k; p.cv = a.cur_v;
   p.mask = a.mask; p.lens = a.kv_seq_len; p.out = a.out; p.mid_o = a.mid_o; p.mid_lse = a.mid_lse;
   p.counters = fused ? a.counters : nullptr;
+  p.block_table = a.block_table;
+  p.table_stride = a.block_table_stride;
+  p.page_shift = a.page_size == 16 ? 4 : a.page_size == 32 ? 5 : a.page_size == 64 ? 6 : 7;
   p.bsz = a.bsz; p.num_q_heads = a.num_q_heads; p.q_len = a.q_len; p.cache_len = a.cache_len;
   p.chunk = pl.chunk; p.num_splits = pl.num_splits;
   p.heads_per_unit = pl.rows_per_group / a.q_len;

@@ -24,6 +24,7 @@ struct KernelParams {
   void* out;
   float* mid_o;
   float* mid_lse;
+  const int32_t* block_table;  // null = contiguous caches; else page index per (sequence, position / page size)
   int32_t* counters;      // one per (sequence, unit, row block) when the merge runs inside stage 1, else null
 
   int32_t bsz;
@@ -42,6 +43,7 @@ struct KernelParams {
   int32_t len_is_i64;
   int32_t mask_vec4;      // every (float) mask row starts 16-byte aligned
   int32_t mask_packed;    // mask holds one bit per (row, tree key): set = attend
+  int32_t page_shift;     // log2(page size) when block_table is set
   float scale_log2;       // sm_scale * log2(e)
 
   int64_t q_stride[3];
@@ -53,6 +55,7 @@ struct KernelParams {
   int64_t out_stride[3];
   int64_t mid_o_stride[4];
   int64_t mid_lse_stride[3];
+  int64_t table_stride;   // block_table elements per sequence
 };
 
 // Launchers implemented in the .hip files. Each returns a fta_status.

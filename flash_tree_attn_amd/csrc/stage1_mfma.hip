@@ -144,6 +144,24 @@ __device__ __forceinline__ f32x4 load_b128_device(const void* ptr) {
   return v;
 }
 __device__ __forceinline__ void settle(f32x4& a) { asm volatile("" : "+v"(a)); }
+// Scalar (wave-uniform) 32-bit loads of N block-table entries, requested together and
+// waited for inside the same statement: the compiler would use vector loads (whose wait
+// drains the tile requests in flight behind them), and a scalar register still in
+// flight must not be visible to it, since it may move registers at will.
+__device__ __forceinline__ void scalar_load_one(const int32_t* p0, int& a0) {
+  asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=&s"(a0) : "s"(p0) : "memory");
+}
+__device__ __forceinline__ void scalar_load_pair(const int32_t* p0, const int32_t* p1, int& a0, int& a1) {
+  asm volatile("s_load_dword %0, %2, 0x0\n\ts_load_dword %1, %3, 0x0\n\ts_waitcnt lgkmcnt(0)"
+               : "=&s"(a0), "=&s"(a1) : "s"(p0), "s"(p1) : "memory");
+}
+__device__ __forceinline__ void scalar_load_quad(const int32_t* p0, const int32_t* p1, const int32_t* p2, const int32_t* p3,
+                                                 int& a0, int& a1, int& a2, int& a3) {
+  asm volatile("s_load_dword %0, %4, 0x0\n\ts_load_dword %1, %5, 0x0\n\ts_load_dword %2, %6, 0x0\n\t"
+               "s_load_dword %3, %7, 0x0\n\ts_waitcnt lgkmcnt(0)"
+               : "=&s"(a0), "=&s"(a1), "=&s"(a2), "=&s"(a3) : "s"(p0), "s"(p1), "s"(p2), "s"(p3) : "memory");
+}
+
 template <int N>
 __device__ __forceinline__ void wait_lgkm(u32x4& a) {
   asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(a) : "n"(N));
@@ -164,7 +182,7 @@ __device__ __forceinline__ void static_for(F&& f) {
 
 // NSK >= 2: K of tile t+1 is read during iteration t and must have been requested an
 // iteration earlier.
-template <typename T, int D, int QB, int NW, int NSK, bool PIPE>
+template <typename T, int D, int QB, int NW, int NSK, bool PIPE, bool PAGED>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(QB == 1 ? 2 : 1, QB == 1 ? 2 : 1)))
 stage1_mfma_kernel(const KernelParams p) {
   using M = Mfma<T>;
@@ -213,8 +231,14 @@ stage1_mfma_kernel(const KernelParams p) {
   const bool wave_active = wave_row0 < p.rows;
   const float c = p.scale_log2;
 
-  const char* kbase = reinterpret_cast<const char*>(static_cast<const T*>(p.k) + b * p.k_stride[0] + cache_head * p.k_stride[1]);
-  const char* vbase = reinterpret_cast<const char*>(static_cast<const T*>(p.v) + b * p.v_stride[0] + cache_head * p.v_stride[1]);
+  // Contiguous caches: base of this sequence's and head's stream. Paged caches: base of
+  // the head inside page 0; the page term comes from the block table per 1 KiB block.
+  constexpr bool paged = PAGED;   // the host picks the instantiation by p.block_table
+  const char* kbase = reinterpret_cast<const char*>(static_cast<const T*>(p.k) + (paged ? 0 : b * p.k_stride[0]) + cache_head * p.k_stride[1]);
+  const char* vbase = reinterpret_cast<const char*>(static_cast<const T*>(p.v) + (paged ? 0 : b * p.v_stride[0]) + cache_head * p.v_stride[1]);
+  const int32_t* table = paged ? p.block_table + b * p.table_stride : nullptr;
+  const int page_mask = (1 << p.page_shift) - 1;
+  const int64_t k_page_bytes = p.k_stride[0] * 2, v_page_bytes = p.v_stride[0] * 2;
   const char* ckbase = reinterpret_cast<const char*>(static_cast<const T*>(p.ck) + b * p.ck_stride[0] + cur_head * p.ck_stride[1]);
   const char* cvbase = reinterpret_cast<const char*>(static_cast<const T*>(p.cv) + b * p.cv_stride[0] + cur_head * p.cv_stride[1]);
 
@@ -251,15 +275,53 @@ stage1_mfma_kernel(const KernelParams p) {
   const uint32_t v_lane_off = static_cast<uint32_t>(ld_rib * p.v_stride[2] * 2 + ld_chunk * 16);
   const int64_t k_row_bytes = p.k_stride[2] * 2, v_row_bytes = p.v_stride[2] * 2;
 
+  // Paged caches: the page of each of this wave's 1 KiB blocks (RPB consecutive positions,
+  // never straddling a page) comes from the block table with wave-uniform (scalar) loads.
+  // The entries of the NEXT cache tile are requested when a tile goes out, so that the
+  // lookup sits in the slack before the barrier: sync_point fetches them before it waits
+  // for the barrier, the tile request after the barrier picks them up.
+  int page_of[kLoadsPerTensor];
+  int pages_for_tile = -1;   // cache tile whose pages `page_of` holds
+  auto load_pages = [&](int ct) __attribute__((always_inline)) {
+    const int32_t* ent[kLoadsPerTensor];
+#pragma unroll
+    for (int i = 0; i < kLoadsPerTensor; ++i) {
+      const int key = min(kv_start + ct * kKeyTile + (i * NW + wave) * RPB, p.cache_len - 1);
+      ent[i] = table + (key >> p.page_shift);
+    }
+    static_assert(kLoadsPerTensor == 1 || kLoadsPerTensor % 2 == 0, "entries are fetched singly, in pairs or in fours");
+    if constexpr (kLoadsPerTensor == 1) {
+      scalar_load_one(ent[0], page_of[0]);
+    } else if constexpr (kLoadsPerTensor % 4 == 0) {
+#pragma unroll
+      for (int i = 0; i < kLoadsPerTensor; i += 4)
+        scalar_load_quad(ent[i], ent[i + 1], ent[i + 2], ent[i + 3], page_of[i], page_of[i + 1], page_of[i + 2], page_of[i + 3]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < kLoadsPerTensor; i += 2) scalar_load_pair(ent[i], ent[i + 1], page_of[i], page_of[i + 1]);
+    }
+    pages_for_tile = ct;
+  };
   auto issue_full_tile = [&](int t) __attribute__((always_inline)) {
     char* kst = smem + (t % NSK) * TL::kTileBytes;
     char* vst = smem + kVRing + (t % NSV) * TL::kTileBytes;
     const int key0 = kv_start + (t - tree_tiles) * kKeyTile;
+    if constexpr (paged) {
+      if (pages_for_tile != t - tree_tiles) load_pages(t - tree_tiles);   // not fetched ahead (first tiles of a split)
+    }
 #pragma unroll
     for (int i = 0; i < kLoadsPerTensor; ++i) {
       const int blk = i * NW + wave;
-      const char* ksrc = kbase + static_cast<int64_t>(key0 + blk * RPB) * k_row_bytes;
-      const char* vsrc = vbase + static_cast<int64_t>(key0 + blk * RPB) * v_row_bytes;
+      const int key = key0 + blk * RPB;
+      const char* ksrc;
+      const char* vsrc;
+      if (paged) {
+        ksrc = kbase + page_of[i] * k_page_bytes + static_cast<int64_t>(key & page_mask) * k_row_bytes;
+        vsrc = vbase + page_of[i] * v_page_bytes + static_cast<int64_t>(key & page_mask) * v_row_bytes;
+      } else {
+        ksrc = kbase + static_cast<int64_t>(key) * k_row_bytes;
+        vsrc = vbase + static_cast<int64_t>(key) * v_row_bytes;
+      }
       __builtin_amdgcn_global_load_lds((const FTA_GLOBAL void*)(ksrc + k_lane_off), (FTA_LDS void*)(kst + blk * TL::kBlockPitch), 16, 0, 0);
       __builtin_amdgcn_global_load_lds((const FTA_GLOBAL void*)(vsrc + v_lane_off), (FTA_LDS void*)(vst + blk * TL::kBlockPitch), 16, 0, 0);
     }
@@ -280,8 +342,14 @@ stage1_mfma_kernel(const KernelParams p) {
     for (int i = 0; i < kLoadsPerTensor; ++i) {
       const int blk = i * NW + wave;
       const int j = min(key0 + blk * RPB + ld_rib, key_lim - 1);
-      __builtin_amdgcn_global_load_lds((const FTA_GLOBAL void*)(kb_ + j * krb + ld_chunk * 16), (FTA_LDS void*)(kst + blk * TL::kBlockPitch), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((const FTA_GLOBAL void*)(vb_ + j * vrb + ld_chunk * 16), (FTA_LDS void*)(vst + blk * TL::kBlockPitch), 16, 0, 0);
+      int64_t koff = j * krb, voff = j * vrb;
+      if (paged && !tree) {   // per-lane page: clamped rows may sit in another page than the block's first row
+        const int64_t page = table[j >> p.page_shift];
+        koff = page * k_page_bytes + (j & page_mask) * krb;
+        voff = page * v_page_bytes + (j & page_mask) * vrb;
+      }
+      __builtin_amdgcn_global_load_lds((const FTA_GLOBAL void*)(kb_ + koff + ld_chunk * 16), (FTA_LDS void*)(kst + blk * TL::kBlockPitch), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const FTA_GLOBAL void*)(vb_ + voff + ld_chunk * 16), (FTA_LDS void*)(vst + blk * TL::kBlockPitch), 16, 0, 0);
     }
   };
   // Tiles are requested in order. A tile may go out once the stage it lands in is free:
@@ -303,6 +371,10 @@ stage1_mfma_kernel(const KernelParams p) {
   // landed, and everybody is past the reads that k_done / v_done describe), then every
   // tile whose stages have become free is requested.
   auto sync_point = [&](int need, int k_done, int v_done) __attribute__((always_inline)) {
+    if constexpr (paged) {   // pages of the tile that goes out after the barrier (harmless if none does)
+      const int ct = next_issue - tree_tiles;
+      load_pages(ct < 0 ? 0 : ct);
+    }
     if (need >= 0) {
       const int younger = next_issue - 1 - need;   // tiles requested after `need`
       if (younger >= 4) wait_vmcnt<4 * kLoadsPerTile>();
@@ -925,11 +997,11 @@ stage1_mfma_kernel(const KernelParams p) {
 #endif
 }
 
-template <typename T, int D, int QB, int NW, int NS, bool PIPE>
+template <typename T, int D, int QB, int NW, int NS, bool PIPE, bool PAGED>
 int launch(const KernelParams& p, hipStream_t stream) {
   constexpr int kSmem = (PIPE ? 2 * NS + 2 : 2 * NS) * TileLayout<D>::kTileBytes;  // K ring of NS stages + V ring of NS (+ 2)
   static_assert(kSmem <= 160 * 1024, "LDS budget");
-  auto kern = stage1_mfma_kernel<T, D, QB, NW, NS, PIPE>;
+  auto kern = stage1_mfma_kernel<T, D, QB, NW, NS, PIPE, PAGED>;
   if (kSmem > 64 * 1024) {
     // Raising the dynamic-LDS limit is a driver call: once per kernel and device, not per launch.
     static thread_local int configured_device = -1;
@@ -947,14 +1019,14 @@ int launch(const KernelParams& p, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? FTA_OK : FTA_ERR_LAUNCH;
 }
 
-template <typename T>
+template <typename T, bool PAGED>
 int launch_t(const KernelParams& p, int head_dim, hipStream_t stream) {
   if (p.rows_per_wg == 256) {  // 8 waves, pipelined, one workgroup per CU, K ring 3 / V ring 5
-    if (head_dim == 128) return launch<T, 128, 1, 8, 3, true>(p, stream);
-    if (head_dim == 64) return launch<T, 64, 1, 8, 3, true>(p, stream);
+    if (head_dim == 128) return launch<T, 128, 1, 8, 3, true, PAGED>(p, stream);
+    if (head_dim == 64) return launch<T, 64, 1, 8, 3, true, PAGED>(p, stream);
   } else if (p.rows_per_wg == 128) {  // 4 waves, plain, two workgroups per CU, K and V rings of 2
-    if (head_dim == 128) return launch<T, 128, 1, 4, 2, false>(p, stream);
-    if (head_dim == 64) return launch<T, 64, 1, 4, 2, false>(p, stream);
+    if (head_dim == 128) return launch<T, 128, 1, 4, 2, false, PAGED>(p, stream);
+    if (head_dim == 64) return launch<T, 64, 1, 4, 2, false, PAGED>(p, stream);
   }
   return FTA_ERR_UNSUPPORTED;
 }
@@ -967,8 +1039,8 @@ int launch_stage1_mfma(const KernelParams& p, int dtype, int head_dim, void* str
   if (p.k_stride[2] * 2 * 8 > 0x7fffffffLL || p.v_stride[2] * 2 * 8 > 0x7fffffffLL) return FTA_ERR_UNSUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (dtype) {
-    case FTA_F16: return launch_t<_Float16>(p, head_dim, s);
-    case FTA_BF16: return launch_t<__bf16>(p, head_dim, s);
+    case FTA_F16: return p.block_table ? launch_t<_Float16, true>(p, head_dim, s) : launch_t<_Float16, false>(p, head_dim, s);
+    case FTA_BF16: return p.block_table ? launch_t<__bf16, true>(p, head_dim, s) : launch_t<__bf16, false>(p, head_dim, s);
     default: return FTA_ERR_UNSUPPORTED;
   }
 }

@@ -92,20 +92,21 @@ __global__ void __launch_bounds__(256) stage1_shuffle_kernel(const KernelParams 
     const bool tree = t >= cache_tiles;
     const int key0 = tree ? (t - cache_tiles) * kKeyTile : kv_start + t * kKeyTile;
     const int key_lim = tree ? L : kv_end;
+    // tree rows: [batch, head, row]; cache rows: per position through cache_row_offset (paged or not)
     const T* kbase = tree ? static_cast<const T*>(p.ck) + b * p.ck_stride[0] + cur_head * p.ck_stride[1]
-                          : static_cast<const T*>(p.k) + b * p.k_stride[0] + cache_head * p.k_stride[1];
+                          : static_cast<const T*>(p.k) + cache_head * p.k_stride[1];
     const T* vbase = tree ? static_cast<const T*>(p.cv) + b * p.cv_stride[0] + cur_head * p.cv_stride[1]
-                          : static_cast<const T*>(p.v) + b * p.v_stride[0] + cache_head * p.v_stride[1];
-    const int64_t kts = tree ? p.ck_stride[2] : p.k_stride[2];
-    const int64_t vts = tree ? p.cv_stride[2] : p.v_stride[2];
+                          : static_cast<const T*>(p.v) + cache_head * p.v_stride[1];
 
     __syncthreads();  // previous tile fully consumed (also orders the Q staging)
     for (int idx = tid; idx < kKeyTile * (D / kVec); idx += 256) {
       const int j = idx / (D / kVec), c = idx % (D / kVec);
       u32x4 kq = {0, 0, 0, 0}, vq = {0, 0, 0, 0};
       if (key0 + j < key_lim) {
-        kq = *reinterpret_cast<const u32x4*>(kbase + (key0 + j) * kts + c * kVec);
-        vq = *reinterpret_cast<const u32x4*>(vbase + (key0 + j) * vts + c * kVec);
+        const int64_t krow = tree ? (key0 + j) * p.ck_stride[2] : cache_row_offset(p, p.k_stride, b, key0 + j);
+        const int64_t vrow = tree ? (key0 + j) * p.cv_stride[2] : cache_row_offset(p, p.v_stride, b, key0 + j);
+        kq = *reinterpret_cast<const u32x4*>(kbase + krow + c * kVec);
+        vq = *reinterpret_cast<const u32x4*>(vbase + vrow + c * kVec);
       }
       *reinterpret_cast<u32x4*>(Ks + j * S::kKPitch + c * kVec) = kq;
       *reinterpret_cast<u32x4*>(Vs + j * D + c * kVec) = vq;

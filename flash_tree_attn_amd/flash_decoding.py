@@ -111,7 +111,7 @@ def _prepare_mask(mask: torch.Tensor, bsz: int, hq: int, L: int, device) -> torc
 
 
 def build_args(q, k_cache, v_cache, current_k, current_v, mask, kv_seq_len, block_size,
-               max_seq_len_in_batch, sm_scale, kv_group_num, force_splits=0, force_kernel=-1):
+               max_seq_len_in_batch, sm_scale, kv_group_num, force_splits=0, force_kernel=-1, block_tables=None):
     """Validates tensors on the Python side and fills an FtaArgs (without out/scratch).
     Returns (args, keepalive) where keepalive holds every tensor the pointers refer to."""
     if q.dim() != 4:
@@ -122,13 +122,22 @@ def build_args(q, k_cache, v_cache, current_k, current_v, mask, kv_seq_len, bloc
         raise RuntimeError("flash_decoding_attention runs on the GPU only; there is no CPU fallback")
     if q.dtype not in _DTYPES:
         raise ValueError(f"unsupported dtype {q.dtype}")
+    paged = block_tables is not None
     for name, t in (("k_cache", k_cache), ("v_cache", v_cache), ("current_k", current_k), ("current_v", current_v)):
         if t.dim() != 4:
             raise ValueError(f"{name} must be 4-dimensional, got {tuple(t.shape)}")
         if t.dtype != q.dtype or t.device != dev:
             raise ValueError(f"{name} must have q's dtype and device")
-        if t.size(0) != bsz or t.size(3) != D:
+        pool = paged and name.endswith("cache")   # [num_pages, num_kv_heads, page_size, head_dim]
+        if (t.size(0) != bsz and not pool) or t.size(3) != D:
             raise ValueError(f"{name} has shape {tuple(t.shape)}, incompatible with q {tuple(q.shape)}")
+    if paged:
+        if block_tables.dim() != 2 or block_tables.size(0) != bsz or block_tables.dtype != torch.int32 or block_tables.device != dev:
+            raise ValueError("block_tables must be an int32 tensor [bsz, pages per sequence] on q's device")
+        if block_tables.stride(1) != 1 and block_tables.size(1) > 1:
+            block_tables = block_tables.contiguous()
+        if k_cache.shape != v_cache.shape:
+            raise FtaAssertionError("paged k_cache and v_cache must have the same shape")
     hkv = k_cache.size(1)
     if v_cache.size(1) != hkv or hkv * int(kv_group_num) != hq:
         raise ValueError(f"num_heads {hq} != num_kv_heads {hkv} * kv_group_num {kv_group_num}")
@@ -148,7 +157,12 @@ def build_args(q, k_cache, v_cache, current_k, current_v, mask, kv_seq_len, bloc
     a.mask, a.kv_seq_len = mask.data_ptr(), kv_seq_len.data_ptr()
     a.bsz, a.num_q_heads, a.num_kv_heads, a.cur_heads = bsz, hq, hkv, current_k.size(1)
     a.q_len, a.head_dim = L, D
-    a.cache_len, a.v_cache_len = k_cache.size(2), v_cache.size(2)
+    if paged:   # logical capacity per sequence; the pools' dim 2 is the page size
+        a.page_size = k_cache.size(2)
+        a.cache_len = a.v_cache_len = block_tables.size(1) * k_cache.size(2)
+        a.block_table, a.block_table_stride = block_tables.data_ptr(), block_tables.stride(0)
+    else:
+        a.cache_len, a.v_cache_len = k_cache.size(2), v_cache.size(2)
     a.block_size = int(block_size)
     a.max_seq_len_hint = 0 if max_seq_len_in_batch is None else max(int(max_seq_len_in_batch), 1)
     a.dtype = _DTYPES[q.dtype]
@@ -162,7 +176,7 @@ def build_args(q, k_cache, v_cache, current_k, current_v, mask, kv_seq_len, bloc
     a.cv_stride[:] = current_v.stride()[:3]
     a.mask_stride[:] = mask.stride()[:3]
     a.mask_kind = _lib.MASK_PACKED_U64 if mask.dtype == torch.int64 else _lib.MASK_ADDITIVE_F32
-    return a, (q, k_cache, v_cache, current_k, current_v, mask, kv_seq_len)
+    return a, (q, k_cache, v_cache, current_k, current_v, mask, kv_seq_len, block_tables)
 
 
 def plan_for(args: "_lib.FtaArgs", num_cus: int) -> "_lib.FtaPlanOut":
@@ -217,12 +231,12 @@ class PreparedCall:
 
 def prepare(q, k_cache, v_cache, current_k, current_v, mask, kv_seq_len, block_size=64,
             max_seq_len_in_batch=None, output=None, mid_output=None, mid_output_lse=None,
-            sm_scale=None, kv_group_num=1, _force_splits=0, _force_kernel=-1) -> PreparedCall:
+            sm_scale=None, kv_group_num=1, _force_splits=0, _force_kernel=-1, block_tables=None) -> PreparedCall:
     """Validates, plans and allocates once; the returned PreparedCall can be launched
     repeatedly (a decode loop that reuses its buffers pays the Python checks once)."""
     _lib.load()
     args, keep = build_args(q, k_cache, v_cache, current_k, current_v, mask, kv_seq_len, block_size,
-                            max_seq_len_in_batch, sm_scale, kv_group_num, _force_splits, _force_kernel)
+                            max_seq_len_in_batch, sm_scale, kv_group_num, _force_splits, _force_kernel, block_tables)
     bsz, hq, L, D = q.shape
     dev = q.device
     pl = plan_for(args, _num_cus(dev))
@@ -274,6 +288,7 @@ def flash_decoding_attention(
     sm_scale: Optional[float] = None,
     kv_group_num: int = 1,
     *,
+    block_tables: Optional[torch.Tensor] = None,
     _force_splits: int = 0,
     _force_kernel: int = -1,
 ) -> torch.Tensor:
@@ -283,8 +298,12 @@ def flash_decoding_attention(
       q [bsz, num_heads, q_len, head_dim]; k_cache / v_cache [bsz, num_kv_heads, ctx, head_dim];
       current_k / current_v [bsz, num_kv_heads, q_len, head_dim]; mask [q_len, q_len] or
       [bsz, num_heads, q_len, q_len], ADDED to the tree logits; kv_seq_len [bsz].
+    Paged caches (the layout the reference's comments describe, flash_tree_attn.py:17-18,233):
+      pass `block_tables` int32 [bsz, pages per sequence]; k_cache / v_cache are then page pools
+      [num_pages, num_kv_heads, page_size, head_dim] with page_size in {16, 32, 64, 128}, and position
+      j of sequence b is row j % page_size of page block_tables[b, j // page_size].
     Returns [bsz, num_heads, q_len, head_dim] in q's dtype.
     """
     return prepare(q, k_cache, v_cache, current_k, current_v, mask, kv_seq_len, block_size,
                    max_seq_len_in_batch, output, mid_output, mid_output_lse, sm_scale, kv_group_num,
-                   _force_splits, _force_kernel).run()
+                   _force_splits, _force_kernel, block_tables).run()

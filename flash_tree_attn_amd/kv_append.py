@@ -17,7 +17,8 @@ from .flash_decoding import _DTYPES, _check, _rows_ok
 
 def append_accepted_kv(k_cache: torch.Tensor, v_cache: torch.Tensor, current_k: torch.Tensor, current_v: torch.Tensor,
                        accept_idx: torch.Tensor, accept_len: torch.Tensor, kv_seq_len: torch.Tensor,
-                       out_kv_seq_len: Optional[torch.Tensor] = None) -> torch.Tensor:
+                       out_kv_seq_len: Optional[torch.Tensor] = None,
+                       block_tables: Optional[torch.Tensor] = None) -> torch.Tensor:
     """For every sequence b and a < accept_len[b]:
         k_cache[b, :, kv_seq_len[b] + a] = current_k[b, :, accept_idx[b, a]]   (same for v)
     and the returned lengths are kv_seq_len + accept_len (clamped to the cache capacity;
@@ -28,6 +29,9 @@ def append_accepted_kv(k_cache: torch.Tensor, v_cache: torch.Tensor, current_k: 
       current_k / _v      [bsz, num_kv_heads, q_len, head_dim]
       accept_idx          int32 [bsz, max_accept]: tree positions of the accepted path, root first
       accept_len          [bsz], dtype of kv_seq_len (int32 or int64)
+    Paged caches: pass `block_tables` int32 [bsz, pages per sequence]; k_cache / v_cache are then the page
+    pools [num_pages, num_kv_heads, page_size, head_dim] of `flash_decoding_attention(block_tables=...)`,
+    and the capacity of a sequence is pages per sequence * page_size.
     """
     lib = _lib.load()
     dev = k_cache.device
@@ -35,7 +39,16 @@ def append_accepted_kv(k_cache: torch.Tensor, v_cache: torch.Tensor, current_k: 
         raise RuntimeError("append_accepted_kv runs on the GPU only; there is no CPU fallback")
     if k_cache.dim() != 4 or k_cache.shape != v_cache.shape:
         raise ValueError("k_cache / v_cache must be [bsz, num_kv_heads, cache_len, head_dim] and alike")
-    bsz, hkv, cache_len, D = k_cache.shape
+    paged = block_tables is not None
+    _, hkv, cache_len, D = k_cache.shape
+    bsz = current_k.size(0) if current_k.dim() == 4 else -1
+    if paged:
+        if block_tables.dim() != 2 or block_tables.size(0) != bsz or block_tables.dtype != torch.int32 or block_tables.device != dev:
+            raise ValueError("block_tables must be an int32 tensor [bsz, pages per sequence] on the caches' device")
+        if block_tables.stride(1) != 1 and block_tables.size(1) > 1:
+            block_tables = block_tables.contiguous()
+    elif k_cache.size(0) != bsz:
+        raise ValueError("k_cache / v_cache must hold one cache per sequence of current_k")
     if k_cache.dtype not in _DTYPES:
         raise ValueError(f"unsupported dtype {k_cache.dtype}")
     if current_k.shape != current_v.shape or current_k.dim() != 4 or current_k.size(0) != bsz or current_k.size(3) != D:
@@ -71,6 +84,9 @@ def append_accepted_kv(k_cache: torch.Tensor, v_cache: torch.Tensor, current_k: 
     a.kv_seq_len, a.kv_seq_len_out = kv_seq_len.data_ptr(), out.data_ptr()
     a.bsz, a.num_kv_heads, a.q_len, a.head_dim = bsz, hkv, current_k.size(2), D
     a.cache_len, a.max_accept = cache_len, accept_idx.size(1)
+    if paged:
+        a.page_size, a.cache_len = cache_len, block_tables.size(1) * cache_len
+        a.block_table, a.block_table_stride = block_tables.data_ptr(), block_tables.stride(0)
     a.dtype = _DTYPES[k_cache.dtype]
     a.len_dtype = _lib.FTA_I64 if kv_seq_len.dtype == torch.int64 else _lib.FTA_I32
     a.k_stride[:] = k_cache.stride()[:3]

@@ -68,6 +68,13 @@ typedef enum fta_kernel {
  *   out       [bsz, num_q_heads, q_len, head_dim], dtype of q: the FINAL result
  *   mid_o     float32 [bsz, num_q_heads, mid_splits, q_len, head_dim]  (flash_tree_attn.py:276-279)
  *   mid_lse   float32 [bsz, num_q_heads, mid_splits, q_len]            (flash_tree_attn.py:280-281)
+ * Paged caches (the layout the reference's kernel comments and docstring still describe,
+ * flash_tree_attn.py:17-18,233, although its code addresses one contiguous cache per
+ * sequence, :72-73): with block_table given, k_cache / v_cache are page pools
+ *   [num_pages, num_kv_heads, page_size, head_dim]   (k_stride = page, head, position in page)
+ * and position j of sequence b lives in page block_table[b, j / page_size] at row
+ * j % page_size. cache_len is then the logical capacity per sequence
+ * (<= pages per sequence * page_size) and bounds kv_seq_len as before.
  * mid_o / mid_lse are scratch; they may be NULL when the plan has num_splits == 1.
  *   counters  int32 [counter_elems], optional. When given (and the plan reports
  *             counter_elems > 0), fta_decode runs ONE launch: the workgroup that
@@ -90,6 +97,7 @@ typedef struct fta_args {
   float* mid_o;
   float* mid_lse;
   int32_t* counters;
+  const int32_t* block_table; /* NULL = contiguous caches; else int32 [bsz, pages per sequence], see below */
 
   int32_t bsz;
   int32_t num_q_heads;
@@ -108,6 +116,7 @@ typedef struct fta_args {
   int32_t force_kernel;     /* -1 = heuristic; else an fta_kernel */
   int32_t counter_elems;    /* int32 elements behind `counters`, 0 when it is NULL */
   int32_t mask_kind;        /* fta_mask_kind of `mask` */
+  int32_t page_size;        /* positions per page, one of 16, 32, 64, 128; ignored without block_table */
   float sm_scale;
 
   int64_t q_stride[3];      /* batch, head, row */
@@ -119,6 +128,7 @@ typedef struct fta_args {
   int64_t out_stride[3];    /* batch, head, row */
   int64_t mid_o_stride[4];  /* batch, head, split, row */
   int64_t mid_lse_stride[3];/* batch, head, split */
+  int64_t block_table_stride; /* batch stride of block_table */
 } fta_args;
 
 /* What the split heuristic decided for one fta_args (pure host arithmetic). */
@@ -193,21 +203,26 @@ typedef struct fta_append_args {
   const void* accept_len;    /* [bsz], len_dtype */
   const void* kv_seq_len;    /* [bsz], len_dtype */
   void* kv_seq_len_out;      /* [bsz], len_dtype */
+  const int32_t* block_table;/* NULL = contiguous caches; else int32 [bsz, pages per sequence] as in fta_args:
+                                k_cache / v_cache are page pools, k_stride = (page, head, position in page) */
 
   int32_t bsz;
   int32_t num_kv_heads;
   int32_t q_len;
   int32_t head_dim;
-  int32_t cache_len;
+  int32_t cache_len;         /* capacity per sequence (paged: <= pages per sequence * page_size) */
   int32_t max_accept;
   int32_t dtype;             /* fta_dtype */
   int32_t len_dtype;         /* fta_len_dtype of accept_len, kv_seq_len and kv_seq_len_out */
+  int32_t page_size;         /* 16, 32, 64 or 128; ignored without block_table */
+  int32_t reserved;
 
   int64_t k_stride[3];       /* batch, head, position */
   int64_t v_stride[3];
   int64_t ck_stride[3];      /* batch, head, row */
   int64_t cv_stride[3];
   int64_t accept_idx_stride; /* batch stride of accept_idx */
+  int64_t block_table_stride;/* batch stride of block_table */
 } fta_append_args;
 
 /* Validates, then launches on `hip_stream`. Asynchronous; allocates nothing. */

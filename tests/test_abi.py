@@ -52,8 +52,8 @@ def test_header_symbols_exported(fta_lib):
 
 
 def test_struct_layout_matches_header(fta_lib, tmp_path):
-    # 11 pointers, 16 int32 + 1 float (padded to 8), 9 stride arrays (8 of 3 + 1 of 4 int64)
-    assert C.sizeof(_lib.FtaArgs) == 11 * 8 + 18 * 4 + (8 * 3 + 4) * 8
+    # 12 pointers, 18 int32 + 1 float (padded to 8), 9 stride arrays (8 of 3 + 1 of 4 int64), 1 int64
+    assert C.sizeof(_lib.FtaArgs) == 12 * 8 + 20 * 4 + (8 * 3 + 4) * 8 + 8
     assert C.sizeof(_lib.FtaPlanOut) == 10 * 4 + 2 * 8
     # ... and field by field against what a C compiler makes of include/fta.h
     fields = [n for n, _ in _lib.FtaArgs._fields_]

@@ -177,3 +177,31 @@ def test_speculative_loop_decode_append_decode():
             ref_v[b, :, t:t + len(pth)] = cv[b][:, pth]
             ref_lens[b] = t + len(pth)
         assert torch.equal(lens, ref_lens) and torch.equal(k_cache, ref_k) and torch.equal(v_cache, ref_v)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("page_size", [16, 64])
+def test_append_into_paged_caches(page_size):
+    """The same append through a block table: gathering the pages back gives the
+    contiguous result, bit for bit; pool pages of other sequences are untouched."""
+    from flash_tree_attn_amd import append_accepted_kv
+    bsz, hkv, L, D, cap = 3, 2, 10, 128, 128
+    x = make(6, bsz, hkv, L, D, cap, torch.bfloat16, [15, 126, 64], [5, 5, 3], 5)
+    k_ref, v_ref, n_ref = append_accepted_kv_oracle(**x)
+    per_seq = cap // page_size
+    g = torch.Generator().manual_seed(page_size)
+    n_pages = bsz * per_seq + 4
+    tables = torch.randperm(n_pages, generator=g)[: bsz * per_seq].view(bsz, per_seq)
+    to_pool = lambda c: c.view(bsz, hkv, per_seq, page_size, D).permute(0, 2, 1, 3, 4).reshape(bsz * per_seq, hkv, page_size, D)
+    kp = torch.full((n_pages, hkv, page_size, D), 7.0, dtype=torch.bfloat16)
+    vp = torch.full_like(kp, -7.0)
+    kp[tables.view(-1)], vp[tables.view(-1)] = to_pool(x["k_cache"]), to_pool(x["v_cache"])
+    d = {k: v.to(DEV) for k, v in x.items()}
+    kpd, vpd = kp.to(DEV), vp.to(DEV)
+    d["k_cache"], d["v_cache"] = kpd, vpd
+    ret = append_accepted_kv(**d, block_tables=tables.to(torch.int32).to(DEV))
+    from_pool = lambda pool: pool.cpu()[tables.view(-1)].view(bsz, per_seq, hkv, page_size, D).permute(0, 2, 1, 3, 4).reshape(bsz, hkv, cap, D)
+    assert torch.equal(from_pool(kpd), k_ref) and torch.equal(from_pool(vpd), v_ref) and torch.equal(ret.cpu(), n_ref)
+    spare = torch.ones(n_pages, dtype=torch.bool)
+    spare[tables.view(-1)] = False
+    assert bool((kpd.cpu()[spare] == 7.0).all()) and bool((vpd.cpu()[spare] == -7.0).all())

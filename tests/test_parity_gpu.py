@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 import torch
 
-from flash_tree_attn_amd import _lib, flash_decoding_attention
+from flash_tree_attn_amd import FtaAssertionError, _lib, flash_decoding_attention
 from flash_tree_attn_amd.synthetic import CONFIGS, make_inputs
 from flash_tree_attn_amd.tree_mask import additive_mask_from_parents, chain_parents, random_tree_parents
 from oracle.tree_attn_oracle import tree_attention_oracle, two_stage_oracle
@@ -354,6 +354,85 @@ def test_single_launch_merge_matches_two_launches(shape):
     stream = torch.cuda.current_stream().cuda_stream
     buf = fd._counters[(x["q"].device.index, stream)]
     assert int(buf.abs().sum()) == 0
+
+
+def to_pages(x, page_size, seed, spare_pages=3):
+    """Scatters the contiguous caches of `x` into a shuffled page pool; returns
+    (k_pages, v_pages, block_tables). Unused pool pages and the rows past each length
+    hold NaN: they must never reach the result."""
+    k, v = x["k_cache"], x["v_cache"]
+    bsz, hkv, tmax, D = k.shape
+    per_seq = -(-tmax // page_size)
+    n_pages = bsz * per_seq + spare_pages
+    g = torch.Generator().manual_seed(seed)
+    perm = torch.randperm(n_pages, generator=g)[: bsz * per_seq].view(bsz, per_seq)
+    kp = torch.full((n_pages, hkv, page_size, D), float("nan"), dtype=k.dtype, device=k.device)
+    vp = torch.full_like(kp, float("nan"))
+    for b in range(bsz):
+        t_b = int(x["kv_seq_len"][b])
+        for pg in range(per_seq):
+            lo, hi = pg * page_size, min((pg + 1) * page_size, tmax, t_b)
+            if hi > lo:
+                kp[perm[b, pg], :, : hi - lo] = k[b, :, lo:hi]
+                vp[perm[b, pg], :, : hi - lo] = v[b, :, lo:hi]
+    return kp, vp, perm.to(torch.int32).to(k.device)
+
+
+@pytest.mark.parametrize("page_size", [16, 32, 64, 128])
+@pytest.mark.parametrize("shape", [
+    # bsz hq hkv  L   D   tmax  dtype           lens              splits
+    (3, 16, 4, 64, 128, 1000, torch.bfloat16, [1000, 517, 63], 0),     # 256 rows: pipelined MFMA variant
+    (2, 8, 2, 16, 128, 700, torch.float16, [700, 129], 3),             # 128-row plain variant, 3 splits
+    (2, 4, 4, 3, 64, 300, torch.float32, [300, 0], 2),                 # shuffle kernel, an empty cache
+])
+def test_paged_caches_equal_contiguous_caches(page_size, shape):
+    """Block-table addressing (flash_tree_attn.py:17-18,233 describe that layout) changes
+    where rows are fetched from, not what is computed: the paged call must reproduce the
+    contiguous call bit for bit, and the oracle within tolerance."""
+    bsz, hq, hkv, L, D, tmax, dtype, lens, splits = shape
+    x = make(81, bsz, hq, hkv, L, D, tmax, dtype, lens)
+    ref = oracle(x)
+    # the same length cap for both calls, so that both cut the same chunks (the paged
+    # capacity is a whole number of pages)
+    out = run(x, _force_splits=splits, max_seq_len_in_batch=tmax)
+    kp, vp, tables = to_pages(x, page_size, seed=page_size)
+    xp = dict(x, k_cache=kp, v_cache=vp)
+    out_paged = run(xp, _force_splits=splits, block_tables=tables, max_seq_len_in_batch=tmax)
+    check(out_paged, ref, dtype)
+    assert torch.equal(out_paged, out)
+
+
+def test_paged_pool_beyond_4_gib():
+    """Page offsets are 64-bit: the pages in use sit at the far end of a 5 GiB pool."""
+    bsz, hq, hkv, L, D, tmax, page = 2, 16, 8, 8, 128, 2048, 16
+    x = make(83, bsz, hq, hkv, L, D, tmax, torch.bfloat16, [2048, 999])
+    page_bytes = hkv * page * D * 2
+    n_pages = (5 << 30) // page_bytes
+    kp = torch.empty((n_pages, hkv, page, D), dtype=torch.bfloat16, device=DEV)
+    vp = torch.empty_like(kp)
+    per_seq = tmax // page
+    g = torch.Generator().manual_seed(7)
+    tables = (n_pages - 1 - torch.randperm(bsz * per_seq, generator=g)).view(bsz, per_seq)
+    for b in range(bsz):
+        kp[tables[b]] = x["k_cache"][b].view(hkv, per_seq, page, D).transpose(0, 1)
+        vp[tables[b]] = x["v_cache"][b].view(hkv, per_seq, page, D).transpose(0, 1)
+    assert int(tables.min()) * page_bytes > (4 << 30)
+    out = run(dict(x, k_cache=kp, v_cache=vp), block_tables=tables.to(torch.int32).to(DEV))
+    check(out, oracle(x), torch.bfloat16)
+    assert torch.equal(out, run(x))
+
+
+def test_paged_argument_errors():
+    x = make(82, 2, 4, 2, 8, 128, 128, torch.float16, [128, 5])
+    kp, vp, tables = to_pages(x, 32, seed=1)
+    xp = dict(x, k_cache=kp, v_cache=vp)
+    with pytest.raises(ValueError):
+        run(xp, block_tables=tables.long())                       # must be int32
+    with pytest.raises(ValueError):
+        run(xp, block_tables=tables[:1])                          # one row per sequence
+    bad = dict(x, k_cache=kp[:, :, :24].contiguous(), v_cache=vp[:, :, :24].contiguous())
+    with pytest.raises(FtaAssertionError):
+        run(bad, block_tables=tables)                             # page size 24 is not a block size
 
 
 # ---------------------------------------------------------------- size-independent properties
