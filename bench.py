@@ -3,7 +3,8 @@
 
 A step is one call of `flash_decoding_attention` (stage 1 + LSE merge) on one batch of
 synthetic input already resident in HBM. Steps rotate over several independent KV-cache
-sets so the footprint exceeds the 256 MB Infinity Cache. Prints ONE JSON line:
+sets so the footprint exceeds the 256 MB Infinity Cache. Before the warm-up steps the
+call runs untimed for --settle-ms so that the card's clocks have settled. Prints ONE JSON line:
 value = achieved GB/s over the whole call (algorithmic bytes / time per call),
 `roofline` = the dominant kernel (stage 1) timed alone with HIP events on the launch
 stream, `cpu_baseline` = the fp32 PyTorch eager oracle on the host cores (a bounded
@@ -25,11 +26,17 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=500)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--settle-ms", type=float, default=150.0,
+                    help="run the call untimed for this long before the warm-up steps: the card raises its clocks over the "
+                         "first tens of milliseconds of load (a 110 us call measures 102 us once they have settled)")
     ap.add_argument("--config", default="cfg3_gqa_8b_bf16", help="workload name (flash_tree_attn_amd.synthetic.CONFIGS)")
     ap.add_argument("--kv-sets", type=int, default=0, help="independent KV caches to rotate over (0 = enough for >1 GiB)")
     ap.add_argument("--splits", type=int, default=0, help="pin the split count (0 = heuristic)")
+    ap.add_argument("--op", default="decode", choices=["decode", "append_kv"],
+                    help="decode = the tree-attention call (the headline); append_kv = the accepted-path KV append that follows it")
+    ap.add_argument("--accept", type=int, default=8, help="accepted tree rows per sequence for --op append_kv")
     ap.add_argument("--paged", type=int, default=0, metavar="PAGE",
                     help="run on paged caches: pages of PAGE positions (16/32/64/128), shuffled in one pool, with a block table")
     ap.add_argument("--packed-mask", action="store_true", help="pass the tree mask as packed bit words instead of float32")
@@ -88,6 +95,53 @@ def cpu_baseline(cfg, x, budget_s):
     }
 
 
+def bench_append(args, cfg, dev):
+    """Times the accepted-path KV append at the workload's shapes: `--accept` rows of the
+    tree per sequence go to the end of each cache; lengths are written out of place so
+    that every step does the same work. Checked against the CPU oracle first."""
+    import torch
+    from flash_tree_attn_amd import append_accepted_kv
+    from flash_tree_attn_amd.synthetic import make_inputs
+    from oracle.kv_append_oracle import append_accepted_kv_oracle
+
+    x = make_inputs(cfg, seed=0, device=dev, gen_device=dev, kv_sets=1)
+    n_acc = min(args.accept, cfg.q_len)
+    g = torch.Generator().manual_seed(0)
+    idx = torch.stack([torch.randperm(cfg.q_len, generator=g)[:n_acc].sort().values for _ in range(cfg.bsz)]).to(torch.int32).to(dev)
+    acc = torch.full((cfg.bsz,), n_acc, dtype=torch.int64, device=dev)
+    lens = (x["kv_seq_len"] - n_acc).clamp_(min=0)
+    out_lens = torch.empty_like(lens)
+    small = slice(0, min(cfg.bsz, 2))   # oracle check on two sequences
+    kc, vc = x["k_cache"][small].clone(), x["v_cache"][small].clone()
+    ref = append_accepted_kv_oracle(kc, vc, x["current_k"][small], x["current_v"][small], idx[small], acc[small], lens[small])
+    got_lens = append_accepted_kv(kc, vc, x["current_k"][small], x["current_v"][small], idx[small], acc[small], lens[small].clone())
+    assert torch.equal(kc.cpu(), ref[0]) and torch.equal(vc.cpu(), ref[1]) and torch.equal(got_lens.cpu(), ref[2])
+
+    run = lambda: append_accepted_kv(x["k_cache"], x["v_cache"], x["current_k"], x["current_v"], idx, acc, lens, out_lens)
+    for _ in range(args.warmup):
+        run()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(args.steps):
+        run()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / args.steps
+    esz = x["k_cache"].element_size()
+    nbytes = 2 * 2 * cfg.bsz * cfg.num_kv_heads * n_acc * cfg.head_dim * esz + cfg.bsz * (n_acc * 4 + 24)   # rows read + written, indices, lengths
+    print(json.dumps({
+        "metric": "accepted-path KV append us/call", "value": round(ms * 1e3, 2), "unit": "us", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u8 (row copies)", "data": "synthetic, resident in HBM",
+        "config": {"workload": cfg.name + " / append_kv", "bsz": cfg.bsz, "kv_heads": cfg.num_kv_heads, "head_dim": cfg.head_dim,
+                   "accepted_rows": n_acc, "algorithmic_bytes": nbytes},
+        "roofline": {"bound": "hbm", "kernel": "append_kv", "achieved": round(nbytes / (ms * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 6), "traffic": None,
+                     "note": "launch-bound: one small kernel per call"},
+    }))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -114,6 +168,8 @@ def main():
         print(json.dumps({"copy_calibration": True, "bytes_read_per_copy": nbytes_copy, "bytes_written_per_copy": nbytes_copy,
                           "copies": max(args.steps, 1)}))
         return
+    if args.op == "append_kv":
+        return bench_append(args, cfg, dev)
     esz = torch.empty((), dtype=cfg.dtype).element_size()
     kv_bytes = 2 * cfg.bsz * cfg.num_kv_heads * cfg.cache_len * cfg.head_dim * esz
     kv_sets = args.kv_sets or max(2, min(8, -(-(1 << 30) // kv_bytes)))
@@ -171,6 +227,12 @@ def main():
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / steps  # ms per step
 
+    # settle phase: steady-state clocks before anything is timed (see --settle-ms)
+    t_settle = time.perf_counter()
+    while (time.perf_counter() - t_settle) * 1e3 < args.settle_ms:
+        for i in range(32):
+            calls[i % kv_sets].run()
+        torch.cuda.synchronize()
     for i in range(args.warmup):
         calls[i % kv_sets].run()
     ms = timed("run", args.steps)
@@ -186,7 +248,7 @@ def main():
     result = {
         "metric": "tree-attn us/call + achieved HBM GB/s (% peak), 8B GQA q_len=64 @8K ctx",
         "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms, "us_per_call": ms * 1e3, "pct_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
+        "settle_ms": args.settle_ms, "ms_per_step": ms, "us_per_call": ms * 1e3, "pct_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}[cfg.dtype],
         "data": "synthetic (seed 0, N(0,1) q/k/v, random tree mask), inputs resident in HBM",

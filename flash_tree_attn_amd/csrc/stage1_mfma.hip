@@ -201,13 +201,6 @@ stage1_mfma_kernel(const KernelParams p) {
   constexpr int kVRing = NSK * TL::kTileBytes;       // byte offset of the V ring
 
   extern __shared__ __attribute__((aligned(16))) char smem[];
-#ifdef FTA_DBG_TIMING
-  long long dbg_t[12]; int dbg_n = 0; const long long dbg_c0 = clock64();
-#define FTA_STAMP() do { if (dbg_n < 12) dbg_t[dbg_n++] = wall_clock64(); } while (0)
-#else
-#define FTA_STAMP() do {} while (0)
-#endif
-  FTA_STAMP();
 
   const WorkItem w = decode_work(p, blockIdx.x);
   int b, split, T_b;
@@ -360,9 +353,6 @@ stage1_mfma_kernel(const KernelParams p) {
   auto issue_ready = [&](int k_done, int v_done) __attribute__((always_inline)) {
     while (next_issue < ntiles && next_issue - k_done < NSK && next_issue - v_done < NSV) {
       const int t = next_issue++;
-#ifdef FTA_DBG_NO_DMA
-      if (t >= NSK) continue;
-#endif
       if (t >= tree_tiles && t - tree_tiles < full_tiles) issue_full_tile(t); else issue_edge_tile(t);
     }
   };
@@ -428,10 +418,7 @@ stage1_mfma_kernel(const KernelParams p) {
   constexpr int kKbOff = (32 / RPB) * TL::kBlockPitch, kKsOff = 2 * TL::kChunkStride;
   constexpr int kKFrags = 2 * KS;   // K fragments per tile (one 128-bit read each)
   constexpr int kVFrags = 4 * DB;   // V^T fragments per tile (two transposing reads each)
-#ifndef FTA_PF
-#define FTA_PF 4
-#endif
-  constexpr int kPF = FTA_PF;       // fragments requested ahead of the MFMA that consumes them
+  constexpr int kPF = 4;            // fragments requested ahead of the MFMA that consumes them
 
   // ---- building blocks -------------------------------------------------------------
   // S^T = K Q^T of tile t (fragment queue: kPF reads ahead of the consuming MFMA).
@@ -489,15 +476,11 @@ stage1_mfma_kernel(const KernelParams p) {
       if constexpr (i < NV) {
         constexpr int g = i;
         constexpr int kOff = (g / DB) * kVRowsOff16 + (g % DB) * 4 * TL::kChunkStride;
-#ifndef FTA_DBG_NO_VREAD
         vlo[g] = lds_read_tr16_b64<kOff>(va);
         vhi[g] = lds_read_tr16_b64<kOff + kVRowsOff8>(va);
-#endif
       } else {
         constexpr int f = i - NV;
-#ifndef FTA_DBG_NO_KREAD
         kf[f] = lds_read_b128<(f % 2) * kKbOff + (f / 2) * kKsOff>(ka);
-#endif
       }
     };
     static_for<0, kPF>(issue);
@@ -512,42 +495,26 @@ stage1_mfma_kernel(const KernelParams p) {
         const s16x8 both = __builtin_shufflevector(__builtin_bit_cast(s16x4, vlo[g]), __builtin_bit_cast(s16x4, vhi[g]), 0, 1, 2, 3, 4, 5, 6, 7);
         const Vec8 a = __builtin_bit_cast(Vec8, both);
 #pragma unroll
-#ifndef FTA_DBG_NO_MMA
         for (int qb = 0; qb < QB; ++qb) o[g % DB][qb] = M::mma(a, pf[qb][g / DB], o[g % DB][qb]);
-#else
-        for (int qb = 0; qb < QB; ++qb) o[g % DB][qb][0] += (float)a[0];
-#endif
       } else {
         constexpr int f = i - NV;
         wait_lgkm<kNewerReads>(kf[f]);
         const Vec8 a = __builtin_bit_cast(Vec8, kf[f]);
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb) {
-#ifndef FTA_DBG_NO_MMA
           if constexpr (f / 2 == 0) {
             const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
             s[f % 2][qb] = M::mma(a, qf[qb][f / 2], zero);
           } else {
             s[f % 2][qb] = M::mma(a, qf[qb][f / 2], s[f % 2][qb]);
           }
-#else
-          s[f % 2][qb][f / 2] = (float)a[0];
-#endif
         }
       }
-#ifndef FTA_DBG_NO_LDSREAD
       if constexpr (i + kPF < NSTEP) issue(std::integral_constant<int, i + kPF>{});
-#else
-      if constexpr (i + kPF < NSTEP && i < kPF) issue(std::integral_constant<int, i + kPF>{});
-#endif
       // the vector-ALU work that runs in this MFMA's shadow; the fence keeps the compiler
       // from regrouping the two streams (it would put all MFMAs first)
-#ifndef FTA_DBG_NO_SLICE
       valu_slice(i, std::integral_constant<int, NSTEP>{});
-#endif
-#ifndef FTA_DBG_NO_FENCE
       __builtin_amdgcn_sched_barrier(0);
-#endif
     });
   };
   // Additive mask values of one tree tile in the accumulator layout (lane = query row,
@@ -773,7 +740,6 @@ stage1_mfma_kernel(const KernelParams p) {
     if (!wave_active) return;
   } else {
     // phase A: the tree tiles, one complete step each (scores, masked softmax, P.V twice)
-    FTA_STAMP();
     for (int u = 0; u < tree_tiles; ++u) {
       sync_point(u, u, u);
       if (!wave_active) continue;
@@ -782,7 +748,6 @@ stage1_mfma_kernel(const KernelParams p) {
       softmax_tile(std::true_type{}, sB, pA, true, u * kKeyTile, L, mask_vals);
       pv_with_residue(u, true, sB);
     }
-    FTA_STAMP();
 
     // phase B: fused iterations over the full cache tiles that have a successor
     const int fused_cnt = cache_tiles >= 1 ? min(full_tiles, cache_tiles - 1) : 0;
@@ -819,7 +784,6 @@ stage1_mfma_kernel(const KernelParams p) {
         cur_in_B = false;
       }
     }
-    FTA_STAMP();
     // canonical roles for the tail: current scores in sB, previous P in pA
     bool pv_pending = fused_cnt >= 1;   // P of tile t-1 has not been multiplied yet
     bool prv_masked = false;
@@ -855,7 +819,6 @@ stage1_mfma_kernel(const KernelParams p) {
     if (!wave_active) return;
     if (pv_pending) pv_with_residue(ntiles - 1, prv_masked, sA);
   }
-  FTA_STAMP();
 
   // ---- epilogue
   // One split (of the launch, or of this sequence when the merge runs in this kernel):
@@ -987,14 +950,6 @@ stage1_mfma_kernel(const KernelParams p) {
         }
     }
   }
-#ifdef FTA_DBG_TIMING
-  FTA_STAMP();
-  if (tid == 0 && (blockIdx.x == 0 || blockIdx.x == gridDim.x - 1)) {
-    long long* dst = reinterpret_cast<long long*>(p.mid_lse) + (blockIdx.x == 0 ? 0 : 16);
-    for (int i = 0; i < dbg_n; ++i) dst[i] = dbg_t[i];
-    dst[15] = dbg_n; dst[14] = clock64() - dbg_c0;
-  }
-#endif
 }
 
 template <typename T, int D, int QB, int NW, int NS, bool PIPE, bool PAGED>
