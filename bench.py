@@ -266,6 +266,21 @@ def main():
                      "stage2_us_per_launch": ms_stage2 * 1e3,
                      "mfma_tflops": nflops / (ms_stage1 * 1e-3) / 1e12},
     }
+    # context for the datasheet peak: what a plain device copy of 1 GiB streams on this box (read + write bytes)
+    src = torch.empty(1 << 29, dtype=torch.bfloat16, device=dev).normal_()
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    e0.record(stream)
+    for _ in range(10):
+        dst.copy_(src)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    copy_gbs = 10 * 2 * src.numel() * 2 / (e0.elapsed_time(e1) * 1e-3) / 1e9
+    del src, dst
+    result["measured_copy_gbs"] = round(copy_gbs, 1)
+    result["roofline"]["frac_of_measured_copy"] = round(gbs_s1 / copy_gbs, 4)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(cfg, x, args.cpu_seconds)
     print(json.dumps(result))

@@ -435,6 +435,48 @@ def test_paged_argument_errors():
         run(bad, block_tables=tables)                             # page size 24 is not a block size
 
 
+def _random_case(rng):
+    """One random configuration of everything the entry point accepts."""
+    dtype = [torch.bfloat16, torch.float16, torch.float32][rng.randrange(3)]
+    D = [32, 64, 128, 256][rng.randrange(4)] if dtype == torch.float32 else [64, 128, 128, 128, 32, 256][rng.randrange(6)]
+    hkv = [1, 2, 3, 4][rng.randrange(4)]
+    G = [1, 2, 4, 8][rng.randrange(4)]
+    L = [1, 2, 5, 8, 16, 17, 31, 32, 48, 64, 65, 100][rng.randrange(12)]
+    if G * L > 512:
+        L = 512 // G
+    bsz = rng.randrange(1, 6)
+    tmax = [64, 100, 257, 600, 1500][rng.randrange(5)]
+    lens = [rng.choice([0, 1, tmax, rng.randrange(0, tmax + 1)]) for _ in range(bsz)]
+    splits = rng.choice([0, 0, 1, 2, 3, 7])
+    cur_heads = hkv if rng.random() < 0.7 else hkv * G
+    return dict(dtype=dtype, D=D, hkv=hkv, hq=hkv * G, L=L, bsz=bsz, tmax=tmax, lens=lens, splits=splits, cur_heads=cur_heads,
+                page=rng.choice([0, 0, 16, 32, 64, 128]), packed=rng.random() < 0.4, len32=rng.random() < 0.3,
+                block=rng.choice([16, 32, 64, 128]), shuffle=rng.random() < 0.2)
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_random_configurations_against_the_oracle(seed):
+    """Seeded random draws over dtype, head_dim, GQA factor, tree size, lengths (incl. 0, 1
+    and full), split count, block size, tree heads, paged or contiguous caches, packed or
+    additive mask, int32 or int64 lengths, either stage-1 kernel."""
+    import random
+    from flash_tree_attn_amd.tree_mask import pack_mask
+    c = _random_case(random.Random(1000 + seed))
+    x = make(2000 + seed, c["bsz"], c["hq"], c["hkv"], c["L"], c["D"], c["tmax"], c["dtype"], c["lens"], cur_heads=c["cur_heads"])
+    ref = oracle(x)
+    kw = dict(_force_splits=c["splits"])
+    if c["shuffle"]:
+        kw["_force_kernel"] = _lib.KERNEL_SHUFFLE
+    if c["packed"]:
+        x["mask"] = pack_mask(x["mask"].cpu()).to(DEV)
+    if c["len32"]:
+        x["kv_seq_len"] = x["kv_seq_len"].int()
+    if c["page"]:
+        x["k_cache"], x["v_cache"], kw["block_tables"] = to_pages(x, c["page"], seed)
+    out = run(x, block_size=c["block"], **kw)
+    check(out, ref, c["dtype"])
+
+
 # ---------------------------------------------------------------- size-independent properties
 def test_properties_at_headline_size():
     cfg = CONFIGS["cfg3_gqa_8b_bf16"]
