@@ -171,6 +171,15 @@ __device__ __forceinline__ void wait_lgkm(u32x2& a, u32x2& b) {
   asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
 }
 
+// A wave-uniform pointer, pinned to scalar registers: address arithmetic on it stays on the
+// scalar unit and loads can use the (scalar base + 32-bit lane offset) addressing form.
+__device__ __forceinline__ const char* uniform_ptr(const char* p) {
+  const uint64_t v = reinterpret_cast<uint64_t>(p);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
+  const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
+  return reinterpret_cast<const char*>((static_cast<uint64_t>(hi) << 32) | lo);
+}
+
 // Compile-time loop: f(std::integral_constant<int, I>) for I in [0, N).
 template <int I, int N, typename F>
 __device__ __forceinline__ void static_for(F&& f) {
@@ -295,25 +304,43 @@ stage1_mfma_kernel(const KernelParams p) {
     }
     pages_for_tile = ct;
   };
+  // Ring slots of the next tile to go out (tiles go out in order, so the slots just count up and wrap).
+  int k_slot = 0, v_slot = 0;
+  auto advance_slots = [&]() __attribute__((always_inline)) {
+    k_slot = k_slot + 1 == NSK ? 0 : k_slot + 1;
+    v_slot = v_slot + 1 == NSV ? 0 : v_slot + 1;
+  };
+  const int64_t k_wave_off = static_cast<int64_t>(wave * RPB) * k_row_bytes, v_wave_off = static_cast<int64_t>(wave * RPB) * v_row_bytes;
+  const int64_t k_step = static_cast<int64_t>(NW * RPB) * k_row_bytes, v_step = static_cast<int64_t>(NW * RPB) * v_row_bytes;
+  const char* k_run = uniform_ptr(kbase + static_cast<int64_t>(kv_start) * k_row_bytes + k_wave_off);   // next full tile, this wave's first block
+  const char* v_run = uniform_ptr(vbase + static_cast<int64_t>(kv_start) * v_row_bytes + v_wave_off);
   auto issue_full_tile = [&](int t) __attribute__((always_inline)) {
-    char* kst = smem + (t % NSK) * TL::kTileBytes;
-    char* vst = smem + kVRing + (t % NSV) * TL::kTileBytes;
+    char* kst = smem + k_slot * TL::kTileBytes;
+    char* vst = smem + kVRing + v_slot * TL::kTileBytes;
     const int key0 = kv_start + (t - tree_tiles) * kKeyTile;
     if constexpr (paged) {
       if (pages_for_tile != t - tree_tiles) load_pages(t - tree_tiles);   // not fetched ahead (first tiles of a split)
     }
+    // contiguous caches: full tiles follow each other in memory, so their scalar base just advances;
+    // the blocks of this wave sit a fixed stride apart
+    const char* ktile = k_run;
+    const char* vtile = v_run;
+    if constexpr (!paged) {
+      k_run = uniform_ptr(k_run + kKeyTile * k_row_bytes);
+      v_run = uniform_ptr(v_run + kKeyTile * v_row_bytes);
+    }
 #pragma unroll
     for (int i = 0; i < kLoadsPerTensor; ++i) {
       const int blk = i * NW + wave;
-      const int key = key0 + blk * RPB;
       const char* ksrc;
       const char* vsrc;
       if (paged) {
+        const int key = key0 + blk * RPB;
         ksrc = kbase + page_of[i] * k_page_bytes + static_cast<int64_t>(key & page_mask) * k_row_bytes;
         vsrc = vbase + page_of[i] * v_page_bytes + static_cast<int64_t>(key & page_mask) * v_row_bytes;
       } else {
-        ksrc = kbase + static_cast<int64_t>(key) * k_row_bytes;
-        vsrc = vbase + static_cast<int64_t>(key) * v_row_bytes;
+        ksrc = uniform_ptr(ktile + i * k_step);
+        vsrc = uniform_ptr(vtile + i * v_step);
       }
       __builtin_amdgcn_global_load_lds((const FTA_GLOBAL void*)(ksrc + k_lane_off), (FTA_LDS void*)(kst + blk * TL::kBlockPitch), 16, 0, 0);
       __builtin_amdgcn_global_load_lds((const FTA_GLOBAL void*)(vsrc + v_lane_off), (FTA_LDS void*)(vst + blk * TL::kBlockPitch), 16, 0, 0);
@@ -322,8 +349,8 @@ stage1_mfma_kernel(const KernelParams p) {
   // Ragged / tree tiles: rows past the limit re-read the last valid row (finite data
   // that the -inf logits then ignore) instead of touching padding.
   auto issue_edge_tile = [&](int t) __attribute__((always_inline)) {
-    char* kst = smem + (t % NSK) * TL::kTileBytes;
-    char* vst = smem + kVRing + (t % NSV) * TL::kTileBytes;
+    char* kst = smem + k_slot * TL::kTileBytes;
+    char* vst = smem + kVRing + v_slot * TL::kTileBytes;
     const bool tree = t < tree_tiles;
     const int key0 = tree ? t * kKeyTile : kv_start + (t - tree_tiles) * kKeyTile;
     const int key_lim = tree ? L : kv_end;
@@ -354,6 +381,7 @@ stage1_mfma_kernel(const KernelParams p) {
     while (next_issue < ntiles && next_issue - k_done < NSK && next_issue - v_done < NSV) {
       const int t = next_issue++;
       if (t >= tree_tiles && t - tree_tiles < full_tiles) issue_full_tile(t); else issue_edge_tile(t);
+      advance_slots();
     }
   };
   // One synchronisation point: this wave's share of tile `need` has landed (tiles land in
