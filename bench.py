@@ -41,6 +41,9 @@ def parse():
                     help="run on paged caches: pages of PAGE positions (16/32/64/128), shuffled in one pool, with a block table")
     ap.add_argument("--packed-mask", action="store_true", help="pass the tree mask as packed bit words instead of float32")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--machine-probe", action="store_true",
+                    help="only run the machine characterisation probes (dense MFMA rate and clock, matrix/vector overlap, "
+                         "streaming rate of the HBM -> LDS load pattern) and print them as one JSON line")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run plain device copies of a known size (reference point for rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
@@ -93,6 +96,44 @@ def cpu_baseline(cfg, x, budget_s):
                   f"{t * 1e6 / nseq * cfg.bsz:.0f} us/call extrapolated to the full batch, os.cpu_count()={os.cpu_count()}",
         "us_per_call_extrapolated": t * 1e6 / nseq * cfg.bsz,
     }
+
+
+def machine_probe():
+    """Runs the probes of libfta_probe.so (flash_tree_attn_amd/csrc/machine_probe.hip)."""
+    import ctypes as C
+    from flash_tree_attn_amd.build import PROBE_LIB_PATH
+    if not os.path.exists(PROBE_LIB_PATH):
+        raise ImportError(f"{PROBE_LIB_PATH} is missing: build it with `python -m flash_tree_attn_amd.build`")
+    lib = C.CDLL(PROBE_LIB_PATH)
+    lib.fta_machine_probe.restype = C.c_int
+    lib.fta_machine_probe.argtypes = [C.c_int, C.c_int, C.POINTER(C.c_double)]
+    names = ["mfma_1_wave_per_simd", "mfma_2_waves_per_simd", "fma_1_wave_per_simd", "roles_mfma_wave_plus_fma_wave",
+             "mixed_both_waves_interleave", "stream_hbm_to_lds", "stream_hbm_to_registers"]
+    res = {}
+    for which, name in enumerate(names):
+        out = (C.c_double * 3)()
+        # a first call settles the clocks, the second is reported
+        for _ in range(2):
+            if lib.fta_machine_probe(which, 20 if which < 5 else 10, out) != 0:
+                raise RuntimeError(f"probe {name} failed")
+        ms, mhz, work = out[0], out[1], out[2]
+        entry = {"ms": round(ms, 4), "shader_clock_mhz": round(mhz)}
+        if which in (0, 1, 3, 4):
+            entry["mfma_tflops"] = round(work / (ms * 1e-3) / 1e12, 1)
+        elif which == 2:
+            entry["fma_lane_ops_per_s"] = work / (ms * 1e-3)
+        else:
+            entry["gbs"] = round(work / (ms * 1e-3) / 1e9, 1)
+        res[name] = entry
+    t = lambda n: res[n]["ms"]
+    res["overlap"] = {
+        "roles_over_sum": round(t("roles_mfma_wave_plus_fma_wave") / (t("mfma_1_wave_per_simd") + t("fma_1_wave_per_simd")), 3),
+        "mixed_over_sum": round(t("mixed_both_waves_interleave") / (t("mfma_2_waves_per_simd") + 2 * t("fma_1_wave_per_simd")), 3),
+        "note": "time of the combination over the sum of its parts run alone: 1.0 = matrix and vector time add up, "
+                "max(a,b)/(a+b) = full overlap. 'roles' = one MFMA wave next to one FMA wave on every SIMD; 'mixed' = both "
+                "waves of every SIMD interleave 1 MFMA + 8 FMA (parts: the 2-wave MFMA probe and twice the 1-wave FMA probe)",
+    }
+    print(json.dumps({"machine_probe": res}))
 
 
 def bench_append(args, cfg, dev):
@@ -158,6 +199,8 @@ def main():
     cfg = CONFIGS[args.config]
     dev = "cuda:0"
     torch.cuda.set_device(0)
+    if args.machine_probe:
+        return machine_probe()
     if args.copy_calibration:
         nbytes_copy = 1 << 30
         src = torch.empty(nbytes_copy // 2, dtype=torch.bfloat16, device=dev).normal_()
@@ -243,6 +286,19 @@ def main():
     # the dominant kernel as launched in the timed region: with the merge inside, the call IS that kernel
     ms_stage1 = ms if single_launch else ms_stage1_alone
 
+    # shader clock the card holds under the stage-1 kernel (measurement hook of the library)
+    clock_mhz = None
+    if plan.kernel == _lib.KERNEL_MFMA:
+        lib = _lib.load()
+        clk = torch.zeros(2, dtype=torch.int64, device=dev)
+        lib.fta_debug_clock_buffer(clk.data_ptr())
+        for i in range(8):
+            calls[i % kv_sets].run_stage1()
+        torch.cuda.synchronize()
+        lib.fta_debug_clock_buffer(None)
+        cyc, ticks = (int(v) for v in clk.tolist())
+        clock_mhz = round(cyc / (ticks / 100.0)) if ticks > 0 else None
+
     gbs = nbytes / (ms * 1e-3) / 1e9
     gbs_s1 = nbytes / (ms_stage1 * 1e-3) / 1e9
     result = {
@@ -264,7 +320,7 @@ def main():
                      "us_per_launch": ms_stage1 * 1e3, "single_launch": single_launch,
                      "two_launch_call_us": ms_two * 1e3, "stage1_without_merge_us": ms_stage1_alone * 1e3,
                      "stage2_us_per_launch": ms_stage2 * 1e3,
-                     "mfma_tflops": nflops / (ms_stage1 * 1e-3) / 1e12},
+                     "mfma_tflops": nflops / (ms_stage1 * 1e-3) / 1e12, "shader_clock_mhz_under_kernel": clock_mhz},
     }
     # context for the datasheet peak: what a plain device copy of 1 GiB streams on this box (read + write bytes)
     src = torch.empty(1 << 29, dtype=torch.bfloat16, device=dev).normal_()

@@ -15,7 +15,7 @@ KERNEL_SHUFFLE, KERNEL_MFMA = 0, 1
 
 EXPORTED_SYMBOLS = (
     "fta_abi_version", "fta_strerror", "fta_validate", "fta_plan", "fta_decode", "fta_decode_stage1",
-    "fta_decode_stage2", "fta_device_cus", "fta_append_kv",
+    "fta_decode_stage2", "fta_device_cus", "fta_append_kv", "fta_debug_clock_buffer",
 )
 
 # status -> Python exception class
@@ -96,6 +96,8 @@ def load() -> C.CDLL:
         fn.restype = C.c_int
         fn.argtypes = [C.POINTER(FtaArgs), C.c_void_p]
     lib.fta_device_cus.restype = C.c_int
+    lib.fta_debug_clock_buffer.restype = C.c_int
+    lib.fta_debug_clock_buffer.argtypes = [C.c_void_p]
     lib.fta_append_kv.restype = C.c_int
     lib.fta_append_kv.argtypes = [C.POINTER(FtaAppendArgs), C.c_void_p]
     if lib.fta_abi_version() != ABI_VERSION:

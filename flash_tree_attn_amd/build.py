@@ -14,6 +14,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 LIB_PATH = os.path.join(HERE, "libfta.so")
+PROBE_LIB_PATH = os.path.join(HERE, "libfta_probe.so")   # machine characterisation kernels for `bench.py --machine-probe`
+PROBE_SOURCES = ["machine_probe.hip"]
 SOURCES = ["fta_host.cpp", "stage1_shuffle.hip", "stage1_mfma.hip", "stage2_merge.hip", "append_kv.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -42,15 +44,23 @@ def _compile(src: str) -> str:
     return obj
 
 
-def build(verbose: bool = True) -> str:
-    with ThreadPoolExecutor(max_workers=min(5, len(SOURCES))) as pool:
-        objs = list(pool.map(_compile, SOURCES))
-    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", *objs, "-o", LIB_PATH]
+def _link(objs, path: str) -> None:
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", *objs, "-o", path]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"link failed:\n{res.stderr}")
+
+
+def build(verbose: bool = True) -> str:
+    """Compiles every HIP source: the product library and the machine-probe library."""
+    all_sources = SOURCES + PROBE_SOURCES
+    with ThreadPoolExecutor(max_workers=min(6, len(all_sources))) as pool:
+        objs = list(pool.map(_compile, all_sources))
+    _link(objs[:len(SOURCES)], LIB_PATH)
+    _link(objs[len(SOURCES):], PROBE_LIB_PATH)
     if verbose:
         print(f"built {LIB_PATH}")
+        print(f"built {PROBE_LIB_PATH}")
     return LIB_PATH
 
 

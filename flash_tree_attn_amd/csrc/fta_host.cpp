@@ -174,7 +174,16 @@ int plan(const fta_args& a, int num_cus, fta_plan_out* out) {
 
 extern "C" {
 
+namespace {
+long long* g_clock_out = nullptr;   // see fta_debug_clock_buffer
+}
+
 int fta_abi_version(void) { return FTA_ABI_VERSION; }
+
+int fta_debug_clock_buffer(void* two_int64_on_device) {
+  g_clock_out = static_cast<long long*>(two_int64_on_device);
+  return FTA_OK;
+}
 
 const char* fta_strerror(int status) {
   switch (status) {
@@ -252,6 +261,7 @@ int decode_impl(const fta_args* args, void* hip_stream, int stages) {
   p.mask = a.mask; p.lens = a.kv_seq_len; p.out = a.out; p.mid_o = a.mid_o; p.mid_lse = a.mid_lse;
   p.counters = fused ? a.counters : nullptr;
   p.block_table = a.block_table;
+  p.clock_out = g_clock_out;
   p.table_stride = a.block_table_stride;
   p.page_shift = a.page_size == 16 ? 4 : a.page_size == 32 ? 5 : a.page_size == 64 ? 6 : 7;
   p.bsz = a.bsz; p.num_q_heads = a.num_q_heads; p.q_len = a.q_len; p.cache_len = a.cache_len;

@@ -25,6 +25,7 @@ struct KernelParams {
   float* mid_o;
   float* mid_lse;
   const int32_t* block_table;  // null = contiguous caches; else page index per (sequence, position / page size)
+  long long* clock_out;   // measurement hook: {shader cycles, 100 MHz ticks} of workgroup 0, or null
   int32_t* counters;      // one per (sequence, unit, row block) when the merge runs inside stage 1, else null
 
   int32_t bsz;

@@ -211,6 +211,7 @@ stage1_mfma_kernel(const KernelParams p) {
 
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
+  const long long clk0 = p.clock_out ? clock64() : 0, ref0 = p.clock_out ? wall_clock64() : 0;
   const WorkItem w = decode_work(p, blockIdx.x);
   int b, split, T_b;
   if (!item_by_order(p, w.item, &b, &split, &T_b)) return;
@@ -896,6 +897,11 @@ stage1_mfma_kernel(const KernelParams p) {
         else *lse_dst = lse_own[qb];
       }
     }
+  }
+
+  if (p.clock_out && blockIdx.x == 0 && tid == 0) {   // measurement hook, see fta_debug_clock_buffer
+    p.clock_out[0] = clock64() - clk0;
+    p.clock_out[1] = wall_clock64() - ref0;
   }
 
   // ---- merge inside this launch (flash_tree_attn.py:339-365 without a second kernel).

@@ -228,6 +228,12 @@ typedef struct fta_append_args {
 /* Validates, then launches on `hip_stream`. Asynchronous; allocates nothing. */
 int fta_append_kv(const fta_append_args* args, void* hip_stream);
 
+/* Measurement hook (no counterpart in the reference): with a device buffer of two int64 set, workgroup 0
+ * of every later stage-1 MFMA launch stores there the shader-clock cycles and the 100 MHz reference ticks
+ * it ran for; their ratio is the clock the card held under the kernel (bench.py reports it). NULL (the
+ * default) switches it off. Process-wide; not meant for concurrent use. */
+int fta_debug_clock_buffer(void* two_int64_on_device);
+
 /* Number of compute units of the current HIP device, or a negative fta_status. */
 int fta_device_cus(void);
 
