@@ -28,7 +28,7 @@ def digest(*tensors) -> str:
 
 
 def cfg1():
-    """BASELINE config 1 at seed 0: inputs are re-drawn from the seed by the test
+    """Workload cfg1_plumbing_fp32 at seed 0: inputs are re-drawn from the seed by the test
     (their digest is stored), the expected fp64 output is stored in full."""
     cfg = CONFIGS["cfg1_plumbing_fp32"]
     x = make_inputs(cfg, seed=0)

@@ -132,7 +132,7 @@ def test_decode_without_scratch_or_device_fails_cleanly(fta_lib):
 
 
 CASES = [
-    dict(),                                                                                     # config 3
+    dict(),                                                                                     # cfg3_gqa_8b_bf16
     dict(bsz=4, num_q_heads=32, num_kv_heads=32, cur_heads=32, q_len=26, cache_len=4096, v_cache_len=4096, dtype=_lib.FTA_F16),
     dict(bsz=1, cache_len=131072, v_cache_len=131072),                                          # config 4
     dict(bsz=64, num_q_heads=64, q_len=16, cache_len=32768, v_cache_len=32768),                 # config 5

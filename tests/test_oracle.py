@@ -51,7 +51,7 @@ def test_whole_path_equals_sdpa(seed):
 
 
 def test_chain_tree_is_causal_attention():
-    """Chain tree (BASELINE config 1's mask) == SDPA is_causal on the last L positions."""
+    """Chain tree (the mask of workload cfg1_plumbing_fp32) == SDPA is_causal on the last L positions."""
     q, k, v, ck, cv, _, _ = rand_case(3, bsz=1, hq=2, hkv=2, L=4, D=8, tmax=12)
     lens = torch.tensor([12])
     mask = additive_mask_from_parents(chain_parents(4)).double()

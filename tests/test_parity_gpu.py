@@ -58,7 +58,7 @@ def check(out, ref, dtype):
 
 # ---------------------------------------------------------------- fixtures
 def test_golden_cfg1_fp32_chain():
-    """BASELINE config 1 (bsz 1, 8 MHA heads, D 64, L 4, chain mask, T 256, fp32)."""
+    """Workload cfg1_plumbing_fp32 (bsz 1, 8 MHA heads, D 64, L 4, chain mask, T 256, fp32)."""
     x = make_inputs(CONFIGS["cfg1_plumbing_fp32"], seed=0, device=DEV)
     out = run(x)
     check(out, oracle(x), torch.float32)
@@ -86,7 +86,7 @@ def test_golden_tiny_gqa_ragged(dtype):
         check(out, ref, dtype)
 
 
-# ---------------------------------------------------------------- BASELINE configs 2-5
+# ---------------------------------------------------------------- workloads cfg2 .. cfg5 at full size
 def test_cfg2_medusa_fp16_ragged():
     cfg = CONFIGS["cfg2_medusa_7b_fp16"]
     x = make_inputs(cfg, seed=0, device=DEV)
