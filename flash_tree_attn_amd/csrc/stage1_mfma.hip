@@ -24,10 +24,18 @@
 // for the transposing read) then fall on distinct banks, and every fragment address is
 // a per-lane base plus a compile-time offset.
 //
-// The split that owns the end of the sequence appends the tree block as extra tiles
-// (current_k / current_v with the additive mask), which replaces the eager block and
-// sigmoid merge of flash_tree_attn.py:367-373. Output: the final result (one split)
-// or a normalised fp32 partial plus its log-sum-exp (flash_tree_attn.py:121-144).
+// The split that owns the end of the sequence also runs the tree block, as extra tiles
+// ahead of its cache tiles (current_k / current_v with the additive or bit-packed mask),
+// which replaces the eager block and sigmoid merge of flash_tree_attn.py:367-373.
+// Output: the final result (one split) or a normalised fp32 partial plus its
+// log-sum-exp (flash_tree_attn.py:121-144); with counters, the workgroup that finishes
+// a sequence last merges the partials itself (flash_tree_attn.py:339-365).
+//
+// Two loop variants: 8 waves / 256 rows with a software pipeline (softmax of tile t
+// sliced behind the MFMAs of P.V(t-1) and K.Q(t+1), K ring 3 / V ring 5, one workgroup
+// per CU), and 4 waves / 128 rows with a plain loop and rings of 2 so that two
+// workgroups share a CU. Caches are contiguous per sequence or paged through a block
+// table (a template parameter, so that the contiguous path carries no lookups).
 #include <cstdlib>
 #include <type_traits>
 
