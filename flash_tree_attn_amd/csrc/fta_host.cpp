@@ -92,7 +92,8 @@ int plan(const fta_args& a, int num_cus, fta_plan_out* out) {
   const int row_blocks = static_cast<int>(cdiv(rows, rows_per_wg));
   // Workgroups one CU holds at a time (LDS- and register-bound, see the kernels): the
   // 128-row MFMA variant is built to share a CU with a second workgroup.
-  const int wg_per_cu = (kernel == FTA_KERNEL_MFMA && rows_per_wg == 128) ? 2 : 1;
+  // The shuffle kernel's workgroups (4 waves, ~40 KB of LDS) fit four to a CU.
+  const int wg_per_cu = kernel != FTA_KERNEL_MFMA ? 4 : rows_per_wg == 128 ? 2 : 1;
 
   const int64_t work_items = static_cast<int64_t>(a.bsz) * units * row_blocks;
   const int64_t t_cap = a.max_seq_len_hint > 0 ? std::min(a.max_seq_len_hint, a.cache_len) : a.cache_len;
@@ -110,12 +111,12 @@ int plan(const fta_args& a, int num_cus, fta_plan_out* out) {
   const int64_t target = static_cast<int64_t>(num_cus) * wg_per_cu;
   const int64_t min_chunk = std::max<int64_t>(gran, 4 * kKeyTile);
   const int64_t s_max = std::max<int64_t>(1, std::min<int64_t>(64, std::max<int64_t>(t_cap, 1) / min_chunk));
-  const double fixed_us = wg_per_cu > 1 ? 12.0 : 20.0;   // partly hidden behind the co-resident workgroup
+  const double fixed_us = kernel != FTA_KERNEL_MFMA ? 5.0 : wg_per_cu > 1 ? 12.0 : 20.0;   // partly hidden behind co-resident workgroups
   // per workgroup and 64-key tile, with the CU fully occupied: the pipelined 256-row
   // variant alone on its CU; the plain 128-row variant next to a second workgroup, by
-  // the number of its waves that hold rows; the shuffle kernel by its rows.
+  // the number of its waves that hold rows; the shuffle kernel with four workgroups per CU.
   const int live_waves = std::min(4, static_cast<int>(cdiv(std::min(rows, rows_per_wg), 32)));
-  const double tile_us = kernel != FTA_KERNEL_MFMA ? 0.6 * rows_per_wg : rows_per_wg > 128 ? 2.85 : 1.0 + 0.7 * live_waves;
+  const double tile_us = kernel != FTA_KERNEL_MFMA ? 5.0 : rows_per_wg > 128 ? 2.85 : 1.0 + 0.7 * live_waves;
   const double tree_tiles = 3.0 * cdiv(a.q_len, kKeyTile);
   const double tail_share = a.bsz > 1 ? 0.25 : 0.0;
   const double partial_mb = 4e-6 * a.bsz * a.num_q_heads * a.q_len * a.head_dim;  // MB per split slot

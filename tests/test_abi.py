@@ -172,7 +172,7 @@ def test_plan_properties(fta_lib, kw, cus):
     # one counter per (sequence, unit, row block) where the merge can run inside stage 1
     fusable = pl.num_splits > 1 and pl.kernel == _lib.KERNEL_MFMA
     assert pl.counter_elems == (pl.num_workgroups // pl.num_splits if fusable else 0)
-    slots = cus * (2 if pl.rows_per_wg == 128 else 1)   # the 128-row variant shares a CU with a second workgroup
+    slots = cus * (2 if pl.rows_per_wg == 128 else 1)   # the 128-row variant shares a CU with a second workgroup (MFMA plans only reach here)
     assert pl.single_launch == int(fusable and pl.num_splits <= 2 and pl.num_workgroups <= slots)
 
 
