@@ -27,10 +27,12 @@ inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 int esize(int dtype) { return dtype == FTA_F32 ? 4 : 2; }
 
-bool mfma_eligible(const fta_args& a, int rows) {
+bool mfma_eligible(const fta_args& a) {
   // The MFMA kernel takes row maxima before scaling, which needs a positive scale.
-  return (a.dtype == FTA_F16 || a.dtype == FTA_BF16) && (a.head_dim == 64 || a.head_dim == 128) && rows >= 16 &&
-         a.sm_scale > 0.f;
+  // No lower bound on the rows of a unit: rows past its end are blanked per lane, and a
+  // unit of one row (plain decode) still streams K/V three times faster through the
+  // DMA-fed MFMA kernel than through the shuffle kernel, whose tiles wait on LDS staging.
+  return (a.dtype == FTA_F16 || a.dtype == FTA_BF16) && (a.head_dim == 64 || a.head_dim == 128) && a.sm_scale > 0.f;
 }
 
 // Query heads that share both their cache head and their tree head.
@@ -83,9 +85,9 @@ int plan(const fta_args& a, int num_cus, fta_plan_out* out) {
   const int rows = hpu * a.q_len;
   const int units = a.num_q_heads / hpu;
 
-  int kernel = mfma_eligible(a, rows) ? FTA_KERNEL_MFMA : FTA_KERNEL_SHUFFLE;
+  int kernel = mfma_eligible(a) ? FTA_KERNEL_MFMA : FTA_KERNEL_SHUFFLE;
   if (a.force_kernel >= 0) {
-    if (a.force_kernel == FTA_KERNEL_MFMA && !mfma_eligible(a, rows)) return FTA_ERR_UNSUPPORTED;
+    if (a.force_kernel == FTA_KERNEL_MFMA && !mfma_eligible(a)) return FTA_ERR_UNSUPPORTED;
     kernel = a.force_kernel;
   }
   const int rows_per_wg = kernel == FTA_KERNEL_MFMA ? mfma_rows_per_wg(rows) : 16;

@@ -1,4 +1,6 @@
-// Stage 1, MFMA variant (f16 / bf16, head_dim 64 or 128, >= 16 query rows per unit).
+// Stage 1, MFMA variant (f16 / bf16, head_dim 64 or 128, positive sm_scale; any number of
+// query rows per unit: rows past a unit's end are blanked per lane, and units of a few
+// rows still stream K/V faster through this kernel's load path than the shuffle variant).
 //
 // One workgroup = (batch, unit, split, row block). A unit is the set of query heads
 // that share one cache head (the GQA group) and one tree head, so its

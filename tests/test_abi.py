@@ -167,7 +167,7 @@ def test_plan_properties(fta_lib, kw, cus):
         assert pl.mid_o_elems == pl.mid_lse_elems * a.head_dim
     else:
         assert pl.mid_o_elems == 0 and pl.mid_lse_elems == 0
-    mfma_ok = a.dtype in (_lib.FTA_F16, _lib.FTA_BF16) and a.head_dim in (64, 128) and pl.rows_per_group >= 16
+    mfma_ok = a.dtype in (_lib.FTA_F16, _lib.FTA_BF16) and a.head_dim in (64, 128) and a.sm_scale > 0
     assert pl.kernel == (_lib.KERNEL_MFMA if mfma_ok else _lib.KERNEL_SHUFFLE)
     # one counter per (sequence, unit, row block) where the merge can run inside stage 1
     fusable = pl.num_splits > 1 and pl.kernel == _lib.KERNEL_MFMA

@@ -422,6 +422,33 @@ def test_paged_pool_beyond_4_gib():
     assert torch.equal(out, run(x))
 
 
+@pytest.mark.parametrize("case", [
+    (1, 1, 4, 4, 1, 128, 300, torch.bfloat16, [300], None, 1),       # plain decode, one row per unit
+    (2, 2, 8, 2, 1, 128, 777, torch.float16, [777, 123], None, 3),   # GQA 4, one token: 4 rows
+    (3, 3, 8, 8, 4, 64, 500, torch.bfloat16, [0, 1, 500], None, 2),
+    (4, 2, 8, 1, 1, 64, 1000, torch.float16, None, None, 4),         # GQA 8: 8 rows
+    (5, 2, 6, 2, 5, 128, 650, torch.bfloat16, None, None, 0),        # 15 rows
+    (6, 2, 8, 2, 3, 128, 400, torch.float16, None, 8, 2),            # tree heads = query heads: 3 rows
+    (7, 4, 4, 4, 13, 64, 900, torch.bfloat16, None, None, 0),
+    (8, 2, 8, 2, 2, 128, 4096, torch.bfloat16, [4096, 4000], None, 8),
+])
+def test_units_below_one_mfma_tile(case):
+    """Units of 1-15 query rows (plain decode, tiny trees) take the MFMA kernel with most
+    rows of its tile blanked; the shuffle kernel on the same inputs must agree with the oracle too."""
+    from flash_tree_attn_amd import flash_decoding as fd
+    from flash_tree_attn_amd.tree_mask import pack_mask
+    seed, bsz, hq, hkv, L, D, tmax, dtype, lens, cur_heads, splits = case
+    x = make(seed, bsz, hq, hkv, L, D, tmax, dtype, lens=lens, cur_heads=cur_heads)
+    ref = oracle(x)
+    pc = fd.prepare(x["q"], x["k_cache"], x["v_cache"], x["current_k"], x["current_v"], x["mask"], x["kv_seq_len"], 64,
+                 None, None, None, None, None, x["kv_group_num"])
+    assert pc.plan.kernel == _lib.KERNEL_MFMA and pc.plan.rows_per_group < 16
+    out = run(x, _force_splits=splits)
+    check(out, ref, dtype)
+    check(run(x, _force_splits=splits, _force_kernel=_lib.KERNEL_SHUFFLE), ref, dtype)
+    assert torch.equal(out, run(dict(x, mask=pack_mask(x["mask"].cpu()).to(DEV)), _force_splits=splits))
+
+
 def test_paged_argument_errors():
     x = make(82, 2, 4, 2, 8, 128, 128, torch.float16, [128, 5])
     kp, vp, tables = to_pages(x, 32, seed=1)
