@@ -44,6 +44,10 @@ def parse():
     ap.add_argument("--machine-probe", action="store_true",
                     help="only run the machine characterisation probes (dense MFMA rate and clock, matrix/vector overlap, "
                          "streaming rate of the HBM -> LDS load pattern) and print them as one JSON line")
+    ap.add_argument("--reference-sweep", action="store_true",
+                    help="only run the sweep of the reference's own benchmark (flash_tree_attn.py:442-487: bsz 2, 32 MHA heads, "
+                         "D 128, fp16, q_len 16..128 x context 64..256, K/V passed as slices of one buffer) through the drop-in "
+                         "call, next to an eager torch attention on the GPU, and print the table as one JSON line")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run plain device copies of a known size (reference point for rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
@@ -136,6 +140,63 @@ def machine_probe():
     print(json.dumps({"machine_probe": res}))
 
 
+def reference_sweep(dev):
+    """The reference's in-file benchmark (flash_tree_attn.py:442-487), shape for shape and
+    call for call: Z 2, H 32, HEAD_DIM 128, fp16 normal(0, 0.5) inputs, block 64, the cache
+    and the tree block passed as slices of one [Z, H, N_CTX + q_len, D] buffer, a fresh
+    call of the drop-in function per step (wrapper included, as its `triton` provider
+    does); the `torch` provider is eager masked attention on the GPU over the
+    concatenated keys, as the reference's torch_tree_attention (flash_tree_attn.py:380-397). Median of
+    event-timed batches, in milliseconds like the reference prints."""
+    import torch
+    from flash_tree_attn_amd import flash_decoding_attention
+    from flash_tree_attn_amd.tree_mask import additive_mask_from_parents, random_tree_parents
+    Z, H, D, blk = 2, 32, 128, 64
+    sm_scale = 1.0 / D ** 0.5
+    g = torch.Generator().manual_seed(0)
+
+    def timed(fn, batches=15, per_batch=20):
+        for _ in range(30):
+            fn()
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(batches):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(per_batch):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            ts.append(e0.elapsed_time(e1) / per_batch)
+        return sorted(ts)[len(ts) // 2]
+
+    rows = []
+    for q_len in (16, 32, 64, 128):
+        for n_ctx in (64, 128, 256):
+            q = (torch.randn(Z, H, q_len, D, generator=g) * 0.5).half().to(dev)
+            k = (torch.randn(Z, H, n_ctx + q_len, D, generator=g) * 0.5).half().to(dev)
+            v = (torch.randn(Z, H, n_ctx + q_len, D, generator=g) * 0.5).half().to(dev)
+            mask = additive_mask_from_parents(random_tree_parents(q_len, g), device=dev)
+            lens = torch.tensor([n_ctx] * Z, device=dev)
+            full_mask = torch.cat([torch.zeros(q_len, n_ctx, device=dev), mask], dim=1).half()
+
+            def eager():
+                p = torch.matmul(q, k.transpose(2, 3)) * sm_scale + full_mask
+                return torch.matmul(torch.softmax(p.float(), dim=-1).half(), v)
+
+            def ours():
+                return flash_decoding_attention(q, k[:, :, :n_ctx], v[:, :, :n_ctx], k[:, :, n_ctx:], v[:, :, n_ctx:], mask, lens,
+                                                block_size=blk, sm_scale=sm_scale)
+
+            torch.testing.assert_close(ours().float(), eager().float(), atol=1e-2, rtol=0)   # the reference test's tolerance (flash_tree_attn.py:440)
+            nbytes = (q.numel() + k.numel() + v.numel()) * 2                                 # the reference's byte count (flash_tree_attn.py:484)
+            ms_ours, ms_eager = timed(ours), timed(eager)
+            rows.append({"q_len": q_len, "n_ctx": n_ctx, "ms": round(ms_ours, 5), "torch_eager_ms": round(ms_eager, 5),
+                         "gbs": round(nbytes / ms_ours * 1e-6, 1)})
+    print(json.dumps({"reference_sweep": {"shape": "Z 2, H 32, D 128, fp16, block 64", "timing": "median of 15 batches of 20 calls, "
+                      "each a fresh call of flash_decoding_attention (Python wrapper included)", "rows": rows}}))
+
+
 def bench_append(args, cfg, dev):
     """Times the accepted-path KV append at the workload's shapes: `--accept` rows of the
     tree per sequence go to the end of each cache; lengths are written out of place so
@@ -201,6 +262,8 @@ def main():
     torch.cuda.set_device(0)
     if args.machine_probe:
         return machine_probe()
+    if args.reference_sweep:
+        return reference_sweep(dev)
     if args.copy_calibration:
         nbytes_copy = 1 << 30
         src = torch.empty(nbytes_copy // 2, dtype=torch.bfloat16, device=dev).normal_()

@@ -19,6 +19,7 @@ There is no CPU or eager fallback: CPU tensors and a missing library raise.
 from __future__ import annotations
 
 import ctypes as C
+import threading
 from typing import Optional
 
 import torch
@@ -49,6 +50,16 @@ def _counters_for(device: torch.device, stream: int, elems: int) -> torch.Tensor
     return buf
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
+def _current_stream(index: int) -> int:
+    """Handle of torch's current stream on device `index` (the reference launches on it too)."""
+    if _raw_stream is not None:
+        return _raw_stream(index)
+    return torch.cuda.current_stream(index).cuda_stream
+
+
 def _check(status: int) -> None:
     if status == 0:
         return
@@ -67,7 +78,10 @@ def _rows_ok(t: torch.Tensor) -> bool:
 def _as_rows(t: torch.Tensor) -> torch.Tensor:
     """128-bit row access needs unit inner stride and 16-byte aligned rows; anything
     else is copied once (the reference honours arbitrary strides, flash_tree_attn.py:311-330)."""
-    return t if _rows_ok(t) else t.contiguous()
+    if _rows_ok(t):
+        return t
+    t = t.contiguous()
+    return t if t.data_ptr() % 16 == 0 else t.clone()   # contiguous but at an odd offset of its storage
 
 
 def _num_cus(device: torch.device) -> int:
@@ -199,14 +213,19 @@ class PreparedCall:
         self._ref = C.byref(args)
 
     def _launch(self, fn, single_launch=False):
-        with torch.cuda.device(self._device):
-            stream = torch.cuda.current_stream(self._device).cuda_stream
-            if single_launch and self.plan.counter_elems > 0:
-                buf = _counters_for(self._device, stream, self.plan.counter_elems)
-                self.args.counters, self.args.counter_elems = buf.data_ptr(), buf.numel()
-            else:
-                self.args.counters, self.args.counter_elems = None, 0
-            _check(fn(self._ref, C.c_void_p(stream)))
+        index = self._device.index
+        if index is not None and torch.cuda.current_device() != index:
+            with torch.cuda.device(index):
+                return self._launch(fn, single_launch)
+        stream = _current_stream(torch.cuda.current_device())
+        if single_launch and self.plan.counter_elems > 0:
+            buf = _counters_for(self._device, stream, self.plan.counter_elems)
+            self.args.counters, self.args.counter_elems = buf.data_ptr(), buf.numel()
+        else:
+            self.args.counters, self.args.counter_elems = None, 0
+        status = fn(self._ref, stream)
+        if status:
+            _check(status)
         return self.output
 
     def run(self):
@@ -272,6 +291,89 @@ def prepare(q, k_cache, v_cache, current_k, current_v, mask, kv_seq_len, block_s
     return PreparedCall(args, pl, output, mid_output, mid_output_lse, keep, dev)
 
 
+# ---- repeat calls of the drop-in function --------------------------------------------
+# A decode loop calls flash_decoding_attention with the same shapes, strides and dtypes
+# over and over, and at short contexts the Python checks above cost more than the kernel.
+# The first call with a given signature goes through prepare(); if it needed no copies or
+# conversions, its filled fta_args and plan are kept (per thread), and later calls with
+# the same signature only refresh the pointers, allocate the output and launch. Whatever
+# depends on tensor VALUES stays on the device (lengths, mask, block table), so the
+# signature is: shape, strides, dtype and device of every tensor plus the scalar arguments.
+_fast = threading.local()
+_FAST_MAX_ENTRIES = 128
+
+
+class _FastEntry:
+    __slots__ = ("args", "ref", "plan", "out_shape", "dtype", "device", "index", "mid_o_shape", "mid_lse_shape", "decode")
+
+
+def _sig(t):
+    return None if t is None else (t.shape, t.stride(), t.dtype, t.device)
+
+
+def _fast_key(q, k_cache, v_cache, current_k, current_v, mask, kv_seq_len, block_size, max_seq_len_in_batch, output,
+              mid_output, mid_output_lse, sm_scale, kv_group_num, block_tables, force_splits, force_kernel):
+    return (q.shape, q.stride(), q.dtype, q.device, _sig(k_cache), _sig(v_cache), _sig(current_k), _sig(current_v),
+            _sig(mask), _sig(kv_seq_len), block_size, max_seq_len_in_batch, _sig(output), _sig(mid_output),
+            _sig(mid_output_lse), sm_scale, kv_group_num, _sig(block_tables), force_splits, force_kernel)
+
+
+def _remember(key, pc, originals, user_mid):
+    """Keeps a prepared call for its signature if the kernels read the caller's tensors as they came."""
+    for orig, kept in zip(originals, pc._keep):
+        if orig is None and kept is None:
+            continue
+        if orig is None or kept is None or kept.dtype != orig.dtype or kept.data_ptr() != orig.data_ptr():
+            return   # copied or converted: such calls take the full path every time
+    if pc._device.index is None or user_mid == "partial":
+        return
+    e = _FastEntry()
+    e.args, e.ref, e.plan = pc.args, C.byref(pc.args), pc.plan
+    e.out_shape, e.dtype, e.device, e.index = tuple(pc.output.shape), pc.output.dtype, pc._device, pc._device.index
+    own_mid = pc.plan.num_splits > 1 and not user_mid
+    e.mid_o_shape = tuple(pc.mid_output.shape) if own_mid else None
+    e.mid_lse_shape = tuple(pc.mid_output_lse.shape) if own_mid else None
+    e.decode = pc._lib.fta_decode
+    cache = _fast.__dict__.setdefault("entries", {})
+    if len(cache) >= _FAST_MAX_ENTRIES:
+        cache.clear()
+    cache[key] = e
+
+
+def _run_remembered(e, q, k_cache, v_cache, current_k, current_v, mask, kv_seq_len, output, mid_output, mid_output_lse,
+                    block_tables):
+    """Launch from a remembered signature; None sends the call down the full path."""
+    if torch.cuda.current_device() != e.index:
+        return None
+    if output is None:
+        output = torch.empty(e.out_shape, dtype=e.dtype, device=e.device)
+    a = e.args
+    pq, pk, pv, pck, pcv, pout = (q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), current_k.data_ptr(),
+                                  current_v.data_ptr(), output.data_ptr())
+    if (pq | pk | pv | pck | pcv | pout) & 15:
+        return None   # rows not 16-byte aligned: the full path copies them
+    a.q, a.k_cache, a.v_cache, a.cur_k, a.cur_v, a.out = pq, pk, pv, pck, pcv, pout
+    a.mask, a.kv_seq_len = mask.data_ptr(), kv_seq_len.data_ptr()
+    if block_tables is not None:
+        a.block_table = block_tables.data_ptr()
+    plan = e.plan
+    if plan.num_splits > 1:
+        if e.mid_o_shape is not None:   # scratch of the planned size, from torch's caching allocator
+            mid_output = torch.empty(e.mid_o_shape, dtype=torch.float32, device=e.device)
+            mid_output_lse = torch.empty(e.mid_lse_shape, dtype=torch.float32, device=e.device)
+        a.mid_o, a.mid_lse = mid_output.data_ptr(), mid_output_lse.data_ptr()
+    stream = _current_stream(e.index)
+    if plan.single_launch:
+        buf = _counters_for(e.device, stream, plan.counter_elems)
+        a.counters, a.counter_elems = buf.data_ptr(), buf.numel()
+    else:
+        a.counters, a.counter_elems = None, 0
+    status = e.decode(e.ref, stream)
+    if status:
+        _check(status)
+    return output
+
+
 def flash_decoding_attention(
     q: torch.Tensor,
     k_cache: torch.Tensor,
@@ -304,6 +406,23 @@ def flash_decoding_attention(
       j of sequence b is row j % page_size of page block_tables[b, j // page_size].
     Returns [bsz, num_heads, q_len, head_dim] in q's dtype.
     """
-    return prepare(q, k_cache, v_cache, current_k, current_v, mask, kv_seq_len, block_size,
-                   max_seq_len_in_batch, output, mid_output, mid_output_lse, sm_scale, kv_group_num,
-                   _force_splits, _force_kernel, block_tables).run()
+    key = None
+    try:
+        key = _fast_key(q, k_cache, v_cache, current_k, current_v, mask, kv_seq_len, block_size, max_seq_len_in_batch,
+                        output, mid_output, mid_output_lse, sm_scale, kv_group_num, block_tables, _force_splits, _force_kernel)
+        entry = _fast.__dict__.get("entries", {}).get(key)
+    except (AttributeError, TypeError):   # not tensors / unhashable scalars: let the full path report it
+        entry = None
+    if entry is not None:
+        out = _run_remembered(entry, q, k_cache, v_cache, current_k, current_v, mask, kv_seq_len, output, mid_output,
+                              mid_output_lse, block_tables)
+        if out is not None:
+            return out
+    pc = prepare(q, k_cache, v_cache, current_k, current_v, mask, kv_seq_len, block_size,
+                 max_seq_len_in_batch, output, mid_output, mid_output_lse, sm_scale, kv_group_num,
+                 _force_splits, _force_kernel, block_tables)
+    out = pc.run()
+    if key is not None and entry is None:
+        _remember(key, pc, (q, k_cache, v_cache, current_k, current_v, mask, kv_seq_len, block_tables),
+                  "partial" if (mid_output is None) != (mid_output_lse is None) else mid_output is not None)
+    return out
