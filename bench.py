@@ -34,6 +34,8 @@ def parse():
     ap.add_argument("--config", default="cfg3_gqa_8b_bf16", help="workload name (flash_tree_attn_amd.synthetic.CONFIGS)")
     ap.add_argument("--kv-sets", type=int, default=0, help="independent KV caches to rotate over (0 = enough for >1 GiB)")
     ap.add_argument("--splits", type=int, default=0, help="pin the split count (0 = heuristic)")
+    ap.add_argument("--kernel", default="auto", choices=["auto", "mfma", "shuffle"],
+                    help="pin the stage-1 kernel (auto = the plan's choice); for comparing the two on one workload")
     ap.add_argument("--op", default="decode", choices=["decode", "append_kv"],
                     help="decode = the tree-attention call (the headline); append_kv = the accepted-path KV append that follows it")
     ap.add_argument("--accept", type=int, default=8, help="accepted tree rows per sequence for --op append_kv")
@@ -306,6 +308,7 @@ def main():
                 x["k_cache_paged"], x["v_cache_paged"], x["tables"] = kc, vc, tables
         calls.append(prepare(x["q"], kc, vc, x["current_k"], x["current_v"], mask_arg, x["kv_seq_len"], cfg.block_size,
                              None, None, None, None, x["sm_scale"], cfg.kv_group_num, _force_splits=args.splits,
+                             _force_kernel={"auto": -1, "mfma": _lib.KERNEL_MFMA, "shuffle": _lib.KERNEL_SHUFFLE}[args.kernel],
                              block_tables=tables))
     if args.paged:   # the contiguous copies are no longer needed, except set 0 for the self-check
         x["k_caches"], x["v_caches"] = x["k_caches"][:1], x["v_caches"][:1]

@@ -1,4 +1,4 @@
-"""Seeded synthetic inputs for the five benchmark / parity configurations.
+"""Seeded synthetic inputs for the five benchmark / parity configurations (and two plain-decode shapes).
 
 Values are drawn in fp32 and cast, the tree comes from `tree_mask`, lengths are
 int64 like the reference's test (flash_tree_attn.py:434). Small configurations are
@@ -41,6 +41,9 @@ CONFIGS: Dict[str, Config] = {
     "cfg3_gqa_8b_bf16": Config("cfg3_gqa_8b_bf16", 8, 32, 8, 128, 64, 8192, torch.bfloat16, "full", "random"),
     "cfg4_long_ctx_bf16": Config("cfg4_long_ctx_bf16", 1, 32, 8, 128, 64, 131072, torch.bfloat16, "full", "random"),
     "cfg5_ragged_70b_bf16": Config("cfg5_ragged_70b_bf16", 64, 64, 8, 128, 16, 32768, torch.bfloat16, "loguniform:512:32768", "random"),
+    # units below one MFMA tile (not BASELINE configurations): plain decode, one row per unit, and one token on a GQA-4 model
+    "decode1_mha_fp16": Config("decode1_mha_fp16", 8, 32, 32, 128, 1, 32768, torch.float16, "full", "chain"),
+    "decode1_gqa4_bf16": Config("decode1_gqa4_bf16", 64, 32, 8, 128, 1, 4096, torch.bfloat16, "full", "chain"),
 }
 
 
