@@ -14,11 +14,12 @@ namespace fta {
 // Query rows one MFMA workgroup holds: 256 (8 waves x 32 rows, two waves per SIMD, one
 // workgroup per CU: the K/V rings take most of the LDS) when the unit has more than 128
 // rows, else 128 (4 waves, short rings, two workgroups per CU). FTA_ROWS_PER_WG=128
-// forces the 4-wave variant (tuning only).
-int mfma_rows_per_wg(int rows) {
+// forces the 4-wave variant (tuning only). head_dim 256 only exists as the 4-wave variant:
+// its tiles are twice as large, two K and two V stages fill the LDS of a CU.
+int mfma_rows_per_wg(int rows, int head_dim) {
   if (const char* env = std::getenv("FTA_ROWS_PER_WG"))
     if (std::atoi(env) == 128) return 128;
-  return rows > 128 ? 256 : 128;
+  return rows > 128 && head_dim <= 128 ? 256 : 128;
 }
 
 namespace {
@@ -32,7 +33,8 @@ bool mfma_eligible(const fta_args& a) {
   // No lower bound on the rows of a unit: rows past its end are blanked per lane, and a
   // unit of one row (plain decode) still streams K/V three times faster through the
   // DMA-fed MFMA kernel than through the shuffle kernel, whose tiles wait on LDS staging.
-  return (a.dtype == FTA_F16 || a.dtype == FTA_BF16) && (a.head_dim == 64 || a.head_dim == 128) && a.sm_scale > 0.f;
+  return (a.dtype == FTA_F16 || a.dtype == FTA_BF16) && (a.head_dim == 64 || a.head_dim == 128 || a.head_dim == 256) &&
+         a.sm_scale > 0.f;
 }
 
 // Query heads that share both their cache head and their tree head.
@@ -90,12 +92,12 @@ int plan(const fta_args& a, int num_cus, fta_plan_out* out) {
     if (a.force_kernel == FTA_KERNEL_MFMA && !mfma_eligible(a)) return FTA_ERR_UNSUPPORTED;
     kernel = a.force_kernel;
   }
-  const int rows_per_wg = kernel == FTA_KERNEL_MFMA ? mfma_rows_per_wg(rows) : 16;
+  const int rows_per_wg = kernel == FTA_KERNEL_MFMA ? mfma_rows_per_wg(rows, a.head_dim) : 16;
   const int row_blocks = static_cast<int>(cdiv(rows, rows_per_wg));
   // Workgroups one CU holds at a time (LDS- and register-bound, see the kernels): the
   // 128-row MFMA variant is built to share a CU with a second workgroup.
   // The shuffle kernel's workgroups (4 waves, ~40 KB of LDS) fit four to a CU.
-  const int wg_per_cu = kernel != FTA_KERNEL_MFMA ? 4 : rows_per_wg == 128 ? 2 : 1;
+  const int wg_per_cu = kernel != FTA_KERNEL_MFMA ? 4 : (rows_per_wg == 128 && a.head_dim <= 128) ? 2 : 1;
 
   const int64_t work_items = static_cast<int64_t>(a.bsz) * units * row_blocks;
   const int64_t t_cap = a.max_seq_len_hint > 0 ? std::min(a.max_seq_len_hint, a.cache_len) : a.cache_len;
@@ -118,7 +120,7 @@ int plan(const fta_args& a, int num_cus, fta_plan_out* out) {
   // variant alone on its CU; the plain 128-row variant next to a second workgroup, by
   // the number of its waves that hold rows; the shuffle kernel with four workgroups per CU.
   const int live_waves = std::min(4, static_cast<int>(cdiv(std::min(rows, rows_per_wg), 32)));
-  const double tile_us = kernel != FTA_KERNEL_MFMA ? 5.0 : rows_per_wg > 128 ? 2.85 : 1.0 + 0.7 * live_waves;
+  const double tile_us = kernel != FTA_KERNEL_MFMA ? 5.0 : rows_per_wg > 128 ? 2.85 : (1.0 + 0.7 * live_waves) * (a.head_dim > 128 ? 2.0 : 1.0);
   const double tree_tiles = 3.0 * cdiv(a.q_len, kKeyTile);
   const double tail_share = a.bsz > 1 ? 0.25 : 0.0;
   const double partial_mb = 4e-6 * a.bsz * a.num_q_heads * a.q_len * a.head_dim;  // MB per split slot

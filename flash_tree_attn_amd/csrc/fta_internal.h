@@ -65,6 +65,6 @@ int launch_stage1_mfma(const KernelParams& p, int dtype, int head_dim, void* str
 int launch_stage2_merge(const KernelParams& p, int dtype, int head_dim, void* stream);
 
 // Rows one MFMA workgroup holds for a unit of `rows` query rows (host + device agree on it).
-int mfma_rows_per_wg(int rows);
+int mfma_rows_per_wg(int rows, int head_dim);
 
 }  // namespace fta

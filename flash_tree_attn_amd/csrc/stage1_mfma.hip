@@ -1,4 +1,4 @@
-// Stage 1, MFMA variant (f16 / bf16, head_dim 64 or 128, positive sm_scale; any number of
+// Stage 1, MFMA variant (f16 / bf16, head_dim 64, 128 or 256, positive sm_scale; any number of
 // query rows per unit: rows past a unit's end are blanked per lane, and units of a few
 // rows still stream K/V faster through this kernel's load path than the shuffle variant).
 //
@@ -36,7 +36,8 @@
 // Two loop variants: 8 waves / 256 rows with a software pipeline (softmax of tile t
 // sliced behind the MFMAs of P.V(t-1) and K.Q(t+1), K ring 3 / V ring 5, one workgroup
 // per CU), and 4 waves / 128 rows with a plain loop and rings of 2 so that two
-// workgroups share a CU. Caches are contiguous per sequence or paged through a block
+// workgroups share a CU (head_dim 256 only has this variant, alone on its CU: its tiles are
+// twice as large). Caches are contiguous per sequence or paged through a block
 // table (a template parameter, so that the contiguous path carries no lookups).
 #include <cstdlib>
 #include <type_traits>
@@ -82,10 +83,10 @@ typedef __attribute__((ext_vector_type(8))) short s16x8;
 template <int D>
 struct TileLayout {
   static constexpr int kRowBytes = D * 2;
-  static constexpr int kRowsPerBlock = 1024 / kRowBytes;           // 4 (D=128) or 8 (D=64)
+  static constexpr int kRowsPerBlock = 1024 / kRowBytes;           // 4 (D=128), 8 (D=64), 2 (D=256)
   static constexpr int kChunkStride = 16 * kRowsPerBlock;          // bytes between chunks of one row
   static constexpr int kBlockPitch = 1024 + kChunkStride;          // pad: consecutive blocks shift banks
-  static constexpr int kBlocks = kKeyTile / kRowsPerBlock;         // 16 or 8
+  static constexpr int kBlocks = kKeyTile / kRowsPerBlock;         // 16, 8, 32
   static constexpr int kTileBytes = kBlocks * kBlockPitch;
   static constexpr int kStageBytes = 2 * kTileBytes;               // K tile then V tile
   // byte offset of 16-byte chunk `c` of tile row `r`
@@ -202,7 +203,8 @@ __device__ __forceinline__ void static_for(F&& f) {
 // NSK >= 2: K of tile t+1 is read during iteration t and must have been requested an
 // iteration earlier.
 template <typename T, int D, int QB, int NW, int NSK, bool PIPE, bool PAGED>
-__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(QB == 1 ? 2 : 1, QB == 1 ? 2 : 1)))
+__global__ void __launch_bounds__(NW * 64)
+__attribute__((amdgpu_waves_per_eu((QB == 1 && D <= 128) ? 2 : 1, (QB == 1 && D <= 128) ? 2 : 1)))   // head_dim 256 needs the whole register file
 stage1_mfma_kernel(const KernelParams p) {
   using M = Mfma<T>;
   using Vec8 = typename M::Vec8;
@@ -395,6 +397,12 @@ stage1_mfma_kernel(const KernelParams p) {
       advance_slots();
     }
   };
+  // "All but the loads of the N youngest tiles have landed". The counter holds 63 at most;
+  // a larger allowance (deep rings of many-load tiles) is cut to that, which only waits longer.
+  auto wait_tiles = [&](auto n_c) __attribute__((always_inline)) {
+    constexpr int kAllow = decltype(n_c)::value * kLoadsPerTile;
+    wait_vmcnt<(kAllow < 63 ? kAllow : 63)>();
+  };
   // One synchronisation point: this wave's share of tile `need` has landed (tiles land in
   // request order; `need` < 0 waits for nothing), then the barrier (everybody's share has
   // landed, and everybody is past the reads that k_done / v_done describe), then every
@@ -406,10 +414,10 @@ stage1_mfma_kernel(const KernelParams p) {
     }
     if (need >= 0) {
       const int younger = next_issue - 1 - need;   // tiles requested after `need`
-      if (younger >= 4) wait_vmcnt<4 * kLoadsPerTile>();
-      else if (younger == 3) wait_vmcnt<3 * kLoadsPerTile>();
-      else if (younger == 2) wait_vmcnt<2 * kLoadsPerTile>();
-      else if (younger == 1) wait_vmcnt<kLoadsPerTile>();
+      if (younger >= 4) wait_tiles(std::integral_constant<int, 4>{});
+      else if (younger == 3) wait_tiles(std::integral_constant<int, 3>{});
+      else if (younger == 2) wait_tiles(std::integral_constant<int, 2>{});
+      else if (younger == 1) wait_tiles(std::integral_constant<int, 1>{});
       else wait_vmcnt<0>();
     }
     __builtin_amdgcn_s_barrier();
@@ -419,9 +427,9 @@ stage1_mfma_kernel(const KernelParams p) {
   // The first tiles go out right behind the Q loads, so that both latencies overlap;
   // then wait for Q alone: everything younger is this wave's share of those tiles.
   issue_ready(0, 0);
-  if (next_issue >= 3) wait_vmcnt<3 * kLoadsPerTile>();
-  else if (next_issue == 2) wait_vmcnt<2 * kLoadsPerTile>();
-  else if (next_issue == 1) wait_vmcnt<kLoadsPerTile>();
+  if (next_issue >= 3) wait_tiles(std::integral_constant<int, 3>{});
+  else if (next_issue == 2) wait_tiles(std::integral_constant<int, 2>{});
+  else if (next_issue == 1) wait_tiles(std::integral_constant<int, 1>{});
   else wait_vmcnt<0>();
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb)
@@ -1026,6 +1034,7 @@ int launch_t(const KernelParams& p, int head_dim, hipStream_t stream) {
   } else if (p.rows_per_wg == 128) {  // 4 waves, plain, two workgroups per CU, K and V rings of 2
     if (head_dim == 128) return launch<T, 128, 1, 4, 2, false, PAGED>(p, stream);
     if (head_dim == 64) return launch<T, 64, 1, 4, 2, false, PAGED>(p, stream);
+    if (head_dim == 256) return launch<T, 256, 1, 4, 2, false, PAGED>(p, stream);   // 132 KB of rings: one workgroup per CU
   }
   return FTA_ERR_UNSUPPORTED;
 }

@@ -1,6 +1,6 @@
 // Stage 1, wavefront-shuffle variant: any dtype (f32/f16/bf16), any head_dim in
 // {32,64,128,256}, any number of query rows, any sign of sm_scale. The general
-// fallback: fp32 inputs, head_dim 32 / 256, non-positive sm_scale.
+// fallback: fp32 inputs, head_dim 32, non-positive sm_scale.
 //
 // One workgroup = (batch, unit, split, block of 16 query rows); 4 waves x 4 rows.
 // Each 64-key tile of K and V is staged once in LDS and shared by the 16 rows.

@@ -50,7 +50,7 @@ typedef enum fta_mask_kind {
 /* Which stage-1 kernel a plan selects. */
 typedef enum fta_kernel {
   FTA_KERNEL_SHUFFLE = 0,  /* wavefront-shuffle reductions: any dtype / head_dim / q_len / sign of sm_scale */
-  FTA_KERNEL_MFMA = 1      /* MFMA tiles: f16/bf16, head_dim 64/128, sm_scale > 0; any number of rows */
+  FTA_KERNEL_MFMA = 1      /* MFMA tiles: f16/bf16, head_dim 64/128/256, sm_scale > 0; any number of rows */
 } fta_kernel;
 
 /*

@@ -140,6 +140,10 @@ CASES = [
     dict(bsz=2, cache_len=0, v_cache_len=0),
     dict(bsz=3, cache_len=100, v_cache_len=100, block_size=16),
     dict(bsz=2, cache_len=100000, v_cache_len=100000, block_size=128, max_seq_len_hint=777),
+    dict(head_dim=256),                                                                         # 256 rows per unit at head_dim 256: two row blocks of 128
+    dict(head_dim=256, num_q_heads=8, num_kv_heads=8, cur_heads=8, q_len=1),                    # plain decode at head_dim 256
+    dict(num_q_heads=32, num_kv_heads=32, cur_heads=32, q_len=1),                               # plain decode: one row per unit, MFMA kernel
+    dict(sm_scale=-0.1),                                                                        # the MFMA kernel needs a positive scale
 ]
 
 
@@ -161,18 +165,20 @@ def test_plan_properties(fta_lib, kw, cus):
     hpu = a.num_q_heads // a.num_kv_heads if a.cur_heads == a.num_kv_heads else 1
     assert pl.rows_per_group == hpu * a.q_len
     assert pl.row_blocks == -(-pl.rows_per_group // pl.rows_per_wg)
+    if a.head_dim == 256:
+        assert pl.rows_per_wg in (16, 128)   # no 256-row variant: its rings would not fit the LDS
     assert pl.num_workgroups == a.bsz * (a.num_q_heads // hpu) * pl.row_blocks * pl.num_splits
     if pl.num_splits > 1:
         assert pl.mid_lse_elems == a.bsz * a.num_q_heads * pl.num_splits * a.q_len
         assert pl.mid_o_elems == pl.mid_lse_elems * a.head_dim
     else:
         assert pl.mid_o_elems == 0 and pl.mid_lse_elems == 0
-    mfma_ok = a.dtype in (_lib.FTA_F16, _lib.FTA_BF16) and a.head_dim in (64, 128) and a.sm_scale > 0
+    mfma_ok = a.dtype in (_lib.FTA_F16, _lib.FTA_BF16) and a.head_dim in (64, 128, 256) and a.sm_scale > 0
     assert pl.kernel == (_lib.KERNEL_MFMA if mfma_ok else _lib.KERNEL_SHUFFLE)
     # one counter per (sequence, unit, row block) where the merge can run inside stage 1
     fusable = pl.num_splits > 1 and pl.kernel == _lib.KERNEL_MFMA
     assert pl.counter_elems == (pl.num_workgroups // pl.num_splits if fusable else 0)
-    slots = cus * (2 if pl.rows_per_wg == 128 else 1)   # the 128-row variant shares a CU with a second workgroup (MFMA plans only reach here)
+    slots = cus * (2 if pl.rows_per_wg == 128 and a.head_dim <= 128 else 1)   # the 128-row variant shares a CU with a second workgroup (MFMA plans only reach here)
     assert pl.single_launch == int(fusable and pl.num_splits <= 2 and pl.num_workgroups <= slots)
 
 
