@@ -12,7 +12,7 @@ from typing import Optional
 import torch
 
 from . import _lib
-from .flash_decoding import _DTYPES, _check, _rows_ok
+from .flash_decoding import _DTYPES, _FAST_MAX_ENTRIES, _as_rows, _check, _current_stream, _fast, _rows_ok, _sig
 
 
 def append_accepted_kv(k_cache: torch.Tensor, v_cache: torch.Tensor, current_k: torch.Tensor, current_v: torch.Tensor,
@@ -34,12 +34,35 @@ def append_accepted_kv(k_cache: torch.Tensor, v_cache: torch.Tensor, current_k: 
     and the capacity of a sequence is pages per sequence * page_size.
     """
     lib = _lib.load()
+    # Repeat calls: the filled arguments of a call signature (shape, strides, dtype, device of every
+    # tensor) are kept per thread, as in flash_decoding_attention; a repeat only refreshes the pointers.
+    try:
+        key = ("append", _sig(k_cache), _sig(v_cache), _sig(current_k), _sig(current_v), _sig(accept_idx), _sig(accept_len),
+               _sig(kv_seq_len), _sig(out_kv_seq_len), _sig(block_tables))
+        entry = _fast.__dict__.get("entries", {}).get(key)
+    except (AttributeError, TypeError):
+        key = entry = None
+    if entry is not None and torch.cuda.current_device() == entry[2]:
+        a, ref, index = entry
+        out = kv_seq_len if out_kv_seq_len is None else out_kv_seq_len
+        pk, pv, pck, pcv = k_cache.data_ptr(), v_cache.data_ptr(), current_k.data_ptr(), current_v.data_ptr()
+        if not (pk | pv | pck | pcv) & 15:
+            a.k_cache, a.v_cache, a.cur_k, a.cur_v = pk, pv, pck, pcv
+            a.accept_idx, a.accept_len = accept_idx.data_ptr(), accept_len.data_ptr()
+            a.kv_seq_len, a.kv_seq_len_out = kv_seq_len.data_ptr(), out.data_ptr()
+            if block_tables is not None:
+                a.block_table = block_tables.data_ptr()
+            status = lib.fta_append_kv(ref, _current_stream(index))
+            if status:
+                _check(status)
+            return out
     dev = k_cache.device
     if dev.type != "cuda":
         raise RuntimeError("append_accepted_kv runs on the GPU only; there is no CPU fallback")
     if k_cache.dim() != 4 or k_cache.shape != v_cache.shape:
         raise ValueError("k_cache / v_cache must be [bsz, num_kv_heads, cache_len, head_dim] and alike")
     paged = block_tables is not None
+    tables_given = block_tables
     _, hkv, cache_len, D = k_cache.shape
     bsz = current_k.size(0) if current_k.dim() == 4 else -1
     if paged:
@@ -61,8 +84,8 @@ def append_accepted_kv(k_cache: torch.Tensor, v_cache: torch.Tensor, current_k: 
     for name, t in (("k_cache", k_cache), ("v_cache", v_cache)):
         if not _rows_ok(t):
             raise ValueError(f"{name} needs unit inner stride and 16-byte aligned rows (it is updated in place)")
-    current_k = current_k if _rows_ok(current_k) else current_k.contiguous()
-    current_v = current_v if _rows_ok(current_v) else current_v.contiguous()
+    originals = (current_k, current_v, accept_idx, accept_len, tables_given)
+    current_k, current_v = _as_rows(current_k), _as_rows(current_v)
     if accept_idx.dim() != 2 or accept_idx.size(0) != bsz or accept_idx.dtype != torch.int32 or accept_idx.device != dev:
         raise ValueError("accept_idx must be an int32 tensor [bsz, max_accept] on the caches' device")
     if accept_idx.stride(1) != 1 and accept_idx.size(1) > 1:
@@ -96,4 +119,12 @@ def append_accepted_kv(k_cache: torch.Tensor, v_cache: torch.Tensor, current_k: 
     a.accept_idx_stride = accept_idx.stride(0)
     with torch.cuda.device(dev):
         _check(lib.fta_append_kv(C.byref(a), C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)))
+    used = (current_k, current_v, accept_idx, accept_len, block_tables)
+    if key is not None and entry is None and dev.index is not None and all(
+            (o is None and u is None) or (o is not None and u is not None and o.data_ptr() == u.data_ptr())
+            for o, u in zip(originals, used)):
+        cache = _fast.__dict__.setdefault("entries", {})
+        if len(cache) >= _FAST_MAX_ENTRIES:
+            cache.clear()
+        cache[key] = (a, C.byref(a), dev.index)
     return out

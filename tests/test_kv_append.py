@@ -110,6 +110,33 @@ def test_append_matches_oracle_bit_for_bit(dtype, out_of_place):
 
 
 @pytest.mark.gpu
+def test_repeat_appends_refresh_pointers_only():
+    """The second call with the same signature reuses the remembered arguments: other data,
+    other tensors, same shapes must still match the oracle; non-contiguous index rows (copied
+    by the full path) are never remembered."""
+    from flash_tree_attn_amd import flash_decoding as fd
+    fd._fast.__dict__.pop("entries", None)
+    for seed, lens, acc in ((11, [10, 93, 0], [6, 2, 1]), (12, [0, 1, 90], [1, 6, 6]), (13, [5, 5, 5], [0, 0, 3])):
+        x = make(seed, 3, 2, 16, 128, 96, torch.bfloat16, lens, acc, 6)
+        k, v, n = append_accepted_kv_oracle(**x)
+        gk, gv, gn = gpu_run(x, out_of_place=True)
+        assert torch.equal(gk, k) and torch.equal(gv, v) and torch.equal(gn, n)
+        assert sum(1 for key in fd._fast.entries if key[0] == "append") == 1
+    x = make(14, 3, 2, 16, 128, 96, torch.bfloat16, [10, 20, 30], [2, 2, 2], 6)
+    wide = torch.zeros(3, 12, dtype=torch.int32)
+    wide[:, ::2] = x["accept_idx"]
+    from flash_tree_attn_amd import append_accepted_kv
+    k, v, n = append_accepted_kv_oracle(**x)
+    for _ in range(2):
+        d = {name: t.to(DEV) for name, t in x.items()}
+        d["accept_idx"] = wide.to(DEV)[:, ::2]
+        assert d["accept_idx"].stride(1) == 2
+        gn = append_accepted_kv(**d)
+        assert torch.equal(d["k_cache"].cpu(), k) and torch.equal(d["v_cache"].cpu(), v) and torch.equal(gn.cpu(), n)
+    assert sum(1 for key in fd._fast.entries if key[0] == "append") == 1
+
+
+@pytest.mark.gpu
 def test_append_edge_cases():
     # int32 lengths, head_dim 32 and 256, out-of-range tree positions are dropped but counted,
     # accept_len beyond max_accept and negative lengths are clamped
