@@ -130,7 +130,7 @@ int plan(const fta_args& a, int num_cus, fta_plan_out* out) {
     const double tiles = std::ceil((std::max<int64_t>(t_cap, 1) / static_cast<double>(kKeyTile) + tree_tiles) / cand);
     const double wg_us = fixed_us + tile_us * tiles;
     const double rounds = static_cast<double>(cdiv(work_items * cand, target));
-    const double merge_us = cand > 1 ? 6.0 + cand * partial_mb / 4.0 : 0.0;
+    const double merge_us = cand > 1 ? 6.0 + cand * partial_mb / 2.0 : 0.0;   // written once, read once, at ~4-5 TB/s
     const double cost = (rounds + tail_share) * wg_us + merge_us;
     if (cand == 1 || cost < best * 0.98) {  // a larger count has to win by 2 %
       best = cost;
