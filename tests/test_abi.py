@@ -192,6 +192,21 @@ def test_plan_headline_shape_fills_the_gpu(fta_lib):
     assert pl4.num_workgroups >= 256
 
 
+@pytest.mark.parametrize("kw,splits,chunk", [
+    (dict(bsz=4, num_q_heads=32, num_kv_heads=32, cur_heads=32, q_len=26, cache_len=4096, v_cache_len=4096, dtype=_lib.FTA_F16), 4, 1088),
+    (dict(), 4, 2112),                                                                            # config 3
+    (dict(bsz=1, cache_len=131072, v_cache_len=131072), 32, 4160),                                # config 4
+    (dict(bsz=64, num_q_heads=64, q_len=16, cache_len=32768, v_cache_len=32768), 3, 11008),      # config 5
+    (dict(bsz=32, num_q_heads=32, num_kv_heads=32, cur_heads=32, q_len=128, cache_len=4096, v_cache_len=4096,
+          dtype=_lib.FTA_F16, block_size=128), 1, 4096),                                          # the reference test's shape: one pass
+])
+def test_plan_of_the_measured_workloads(fta_lib, kw, splits, chunk):
+    """The split counts the published measurements were taken with (each the measured optimum
+    or within 2 % of it on a 256-CU part): a change of the cost model that moves them needs new measurements."""
+    st, pl = plan(fta_lib, base_args(**kw))
+    assert st == 0 and (pl.num_splits, pl.chunk) == (splits, chunk)
+
+
 def test_plan_overrides(fta_lib):
     st, pl = plan(fta_lib, base_args(force_splits=3))
     assert st == 0 and pl.num_splits == 3
