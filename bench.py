@@ -21,6 +21,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+MFMA_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 / fp16 MFMA rate (the co-constraint of the headline shape)
 
 
 def parse():
@@ -390,7 +391,9 @@ def main():
                      "us_per_launch": ms_stage1 * 1e3, "single_launch": single_launch,
                      "two_launch_call_us": ms_two * 1e3, "stage1_without_merge_us": ms_stage1_alone * 1e3,
                      "stage2_us_per_launch": ms_stage2 * 1e3,
-                     "mfma_tflops": nflops / (ms_stage1 * 1e-3) / 1e12, "shader_clock_mhz_under_kernel": clock_mhz},
+                     "mfma_tflops": nflops / (ms_stage1 * 1e-3) / 1e12,
+                     "mfma_frac_of_dense_peak": round(nflops / (ms_stage1 * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4),
+                     "shader_clock_mhz_under_kernel": clock_mhz},
     }
     # context for the datasheet peak: what a plain device copy of 1 GiB streams on this box (read + write bytes)
     src = torch.empty(1 << 29, dtype=torch.bfloat16, device=dev).normal_()
