@@ -496,6 +496,34 @@ def test_repeat_calls_take_the_remembered_signature(monkeypatch):
     check(run(dict(x2, q=q_off)), oracle(x2), torch.bfloat16)
 
 
+def test_calls_follow_the_current_stream():
+    """The library launches on torch's current stream (as the reference's Triton launches do):
+    calls issued under `torch.cuda.stream(side)` must be ordered with other work of that stream,
+    on the full path, on the remembered path and with the merge inside stage 1 (whose counter
+    buffer is kept per stream)."""
+    from flash_tree_attn_amd import flash_decoding as fd
+    fd._fast.__dict__.pop("entries", None)
+    x = make(91, 2, 8, 2, 16, 128, 3000, torch.bfloat16, lens=[3000, 2500])
+    ref = oracle(x)
+    pc = fd.prepare(x["q"], x["k_cache"], x["v_cache"], x["current_k"], x["current_v"], x["mask"], x["kv_seq_len"], 64,
+                    None, None, None, None, None, x["kv_group_num"], _force_splits=2)
+    assert pc.plan.single_launch == 1
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    outs = []
+    with torch.cuda.stream(side):
+        scale = torch.full((1,), 2.0, device=DEV, dtype=torch.bfloat16)
+        for _ in range(3):                      # full path once, then the remembered signature
+            q2 = x["q"] * scale                 # produced on the side stream right before the call
+            outs.append(run(dict(x, q=q2), _force_splits=2, sm_scale=0.5 / math.sqrt(128)))
+            outs.append(run(dict(x, q=q2), _force_splits=1, sm_scale=0.5 / math.sqrt(128)) * 1.0)   # consumed on it right after
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    for o in outs:
+        check(o, ref, torch.bfloat16)
+    assert any(k[1] == side.cuda_stream for k in fd._counters)
+
+
 def test_paged_argument_errors():
     x = make(82, 2, 4, 2, 8, 128, 128, torch.float16, [128, 5])
     kp, vp, tables = to_pages(x, 32, seed=1)
