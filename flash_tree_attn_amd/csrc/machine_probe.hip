@@ -186,13 +186,12 @@ int fta_machine_probe(int which, int reps, double* out) {
   hipEvent_t e0, e1;
   if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) return -1;
   for (int i = 0; i < 3; ++i) launch();   // warm-up
-  hipEventRecord(e0, 0);
+  int rc = hipEventRecord(e0, 0) == hipSuccess ? 0 : -1;
   for (int i = 0; i < reps; ++i) launch();
-  hipEventRecord(e1, 0);
-  int rc = 0;
+  if (hipEventRecord(e1, 0) != hipSuccess) rc = -1;
   if (hipEventSynchronize(e1) != hipSuccess || hipGetLastError() != hipSuccess) rc = -1;
   float ms = 0.f;
-  hipEventElapsedTime(&ms, e0, e1);
+  if (hipEventElapsedTime(&ms, e0, e1) != hipSuccess) rc = -1;
   long long clk[2] = {0, 1};
   if (hipMemcpy(clk, b.clocks, sizeof(clk), hipMemcpyDeviceToHost) != hipSuccess) rc = -1;
   out[0] = ms / reps;
@@ -205,12 +204,13 @@ int fta_machine_probe(int which, int reps, double* out) {
     case 2: out[2] = 0.5 * waves * iters * kFmaPerIter * 64.0; break;
     default: out[2] = 2.0 * stream_bytes; break;
   }
-  hipEventDestroy(e0);
-  hipEventDestroy(e1);
-  hipFree(b.sink);
-  hipFree(b.clocks);
-  if (b.kbuf) hipFree(b.kbuf);
-  if (b.vbuf) hipFree(b.vbuf);
+  // teardown: a failure here cannot be acted on, the measurement above stands or falls by rc
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  (void)hipFree(b.sink);
+  (void)hipFree(b.clocks);
+  if (b.kbuf) (void)hipFree(b.kbuf);
+  if (b.vbuf) (void)hipFree(b.vbuf);
   return rc;
 }
 
