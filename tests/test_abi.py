@@ -224,3 +224,35 @@ def test_python_wrapper_rejects_cpu_tensors():
     kv = torch.zeros(1, 2, 16, 64)
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         flash_decoding_attention(q, kv, kv, q, q, torch.zeros(4, 4), torch.tensor([16]))
+
+
+# ---------------------------------------------------------------- the heuristic against measured split sweeps
+def _regrets(fta_lib, fixture):
+    """For every shape of a measured sweep (time of the whole call per forced split count, MI355X,
+    bf16, head_dim 128, tests/golden/split_sweep_*.json): time at the plan's own split count over the
+    best measured time. Counts between two measured ones are interpolated."""
+    import json
+    rows = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", fixture)))
+    out = []
+    for r in rows:
+        st, pl = plan(fta_lib, base_args(bsz=r["bsz"], num_q_heads=r["hq"], num_kv_heads=r["hkv"], cur_heads=r["hkv"], q_len=r["L"],
+                                         cache_len=r["T"], v_cache_len=r["T"]))
+        assert st == 0
+        pts = sorted((int(k), v) for k, v in r["us"].items())
+        s = min(max(pl.num_splits, pts[0][0]), pts[-1][0])
+        lo = max(p for p in pts if p[0] <= s)
+        hi = min(p for p in pts if p[0] >= s)
+        t = lo[1] if hi[0] == lo[0] else lo[1] + (hi[1] - lo[1]) * (s - lo[0]) / (hi[0] - lo[0])
+        out.append(t / min(v for _, v in pts))
+    return out
+
+
+def test_split_heuristic_against_measured_sweeps(fta_lib):
+    """A regression guard for changes of the cost model: on 112 shapes with full-length sequences the
+    plan's split count must stay within 6 % of the best measured one on average (measured: 4 %), on 76
+    shapes with log-uniform lengths within 12 % (measured: 9 %; lengths are not known to the plan)."""
+    uniform = _regrets(fta_lib, "split_sweep_uniform.json")
+    ragged = _regrets(fta_lib, "split_sweep_ragged.json")
+    assert len(uniform) == 112 and len(ragged) == 76
+    assert sum(uniform) / len(uniform) < 1.06 and max(uniform) < 1.40
+    assert sum(ragged) / len(ragged) < 1.12
