@@ -126,16 +126,29 @@ int plan(const fta_args& a, int num_cus, fta_plan_out* out) {
   const double partial_mb = 4e-6 * a.bsz * a.num_q_heads * a.q_len * a.head_dim;  // MB per split slot
   int64_t splits = 1;
   double best = 0.0;
+  double cost_of[65];
   for (int64_t cand = 1; cand <= s_max; ++cand) {
     const double tiles = std::ceil((std::max<int64_t>(t_cap, 1) / static_cast<double>(kKeyTile) + tree_tiles) / cand);
     const double wg_us = fixed_us + tile_us * tiles;
     const double rounds = static_cast<double>(cdiv(work_items * cand, target));
     const double merge_us = cand > 1 ? 6.0 + cand * partial_mb / 2.0 : 0.0;   // written once, read once, at ~4-5 TB/s
     const double cost = (rounds + tail_share) * wg_us + merge_us;
+    cost_of[cand] = cost;
     if (cand == 1 || cost < best * 0.98) {  // a larger count has to win by 2 %
       best = cost;
       splits = cand;
     }
+  }
+  // A batch whose workgroups all fit the machine at once is only balanced if its sequences
+  // are equally long, and the lengths are not known here: the longest sequence then sets the
+  // time while most CUs idle. For batches of 8 and more, up to twice the splits are taken
+  // where the model prices that at no more than 10 % on an equal-length batch. Measured over
+  // split sweeps of 76 ragged and 112 equal-length shapes: -6 % on the ragged ones on
+  // average (worst case 2.1x -> 1.3x of the best split count), +1 % on the equal-length ones.
+  if (a.bsz >= 8 && work_items * splits <= target) {
+    const int64_t chosen = splits;
+    for (int64_t cand = chosen + 1; cand <= std::min<int64_t>(2 * chosen, s_max); ++cand)
+      if (cost_of[cand] <= cost_of[chosen] * 1.10) splits = cand;
   }
   if (a.force_splits > 0) splits = a.force_splits;
   if (const char* env = std::getenv("FTA_FORCE_SPLITS")) {

@@ -249,10 +249,10 @@ def _regrets(fta_lib, fixture):
 
 def test_split_heuristic_against_measured_sweeps(fta_lib):
     """A regression guard for changes of the cost model: on 112 shapes with full-length sequences the
-    plan's split count must stay within 6 % of the best measured one on average (measured: 4 %), on 76
-    shapes with log-uniform lengths within 12 % (measured: 9 %; lengths are not known to the plan)."""
+    plan's split count must stay within 5 % of the best measured one on average (it is at 3.3 %), on 76
+    shapes with log-uniform lengths within 6 % (it is at 3.9 %; lengths are not known to the plan)."""
     uniform = _regrets(fta_lib, "split_sweep_uniform.json")
     ragged = _regrets(fta_lib, "split_sweep_ragged.json")
     assert len(uniform) == 112 and len(ragged) == 76
-    assert sum(uniform) / len(uniform) < 1.06 and max(uniform) < 1.40
-    assert sum(ragged) / len(ragged) < 1.12
+    assert sum(uniform) / len(uniform) < 1.05 and max(uniform) < 1.35
+    assert sum(ragged) / len(ragged) < 1.06 and max(ragged) < 1.40
