@@ -145,7 +145,7 @@ int plan(const fta_args& a, int num_cus, fta_plan_out* out) {
   // where the model prices that at no more than 10 % on an equal-length batch. Measured over
   // split sweeps of 76 ragged and 112 equal-length shapes: -6 % on the ragged ones on
   // average (worst case 2.1x -> 1.3x of the best split count), +1 % on the equal-length ones.
-  if (a.bsz >= 8 && work_items * splits <= target) {
+  if (a.bsz >= 8 && a.head_dim <= 128 && work_items * splits <= target) {   // head_dim 256: the model is not calibrated well enough
     const int64_t chosen = splits;
     for (int64_t cand = chosen + 1; cand <= std::min<int64_t>(2 * chosen, s_max); ++cand)
       if (cost_of[cand] <= cost_of[chosen] * 1.10) splits = cand;
