@@ -38,13 +38,15 @@ _cu_count = {}
 _counters = {}
 
 
-def _counters_for(device: torch.device, stream: int, elems: int) -> torch.Tensor:
+def _counters_for(device: torch.device, stream: int, elems: int) -> Optional[torch.Tensor]:
     """Zeroed int32 counters for the single-launch merge. The kernel leaves them zero
     again, so one buffer per (device, stream) serves every call issued on that stream;
     calls on different streams may overlap in time and get buffers of their own."""
     key = (device.index, stream)
     buf = _counters.get(key)
     if buf is None or buf.numel() < elems:
+        if torch.cuda.is_current_stream_capturing():
+            return None   # no allocation and fill inside a captured graph: the call takes two launches there
         buf = torch.zeros(max(elems, 4096), dtype=torch.int32, device=device)
         _counters[key] = buf
     return buf
@@ -218,8 +220,8 @@ class PreparedCall:
             with torch.cuda.device(index):
                 return self._launch(fn, single_launch)
         stream = _current_stream(torch.cuda.current_device())
-        if single_launch and self.plan.counter_elems > 0:
-            buf = _counters_for(self._device, stream, self.plan.counter_elems)
+        buf = _counters_for(self._device, stream, self.plan.counter_elems) if single_launch and self.plan.counter_elems > 0 else None
+        if buf is not None:
             self.args.counters, self.args.counter_elems = buf.data_ptr(), buf.numel()
         else:
             self.args.counters, self.args.counter_elems = None, 0
@@ -363,8 +365,8 @@ def _run_remembered(e, q, k_cache, v_cache, current_k, current_v, mask, kv_seq_l
             mid_output_lse = torch.empty(e.mid_lse_shape, dtype=torch.float32, device=e.device)
         a.mid_o, a.mid_lse = mid_output.data_ptr(), mid_output_lse.data_ptr()
     stream = _current_stream(e.index)
-    if plan.single_launch:
-        buf = _counters_for(e.device, stream, plan.counter_elems)
+    buf = _counters_for(e.device, stream, plan.counter_elems) if plan.single_launch else None
+    if buf is not None:
         a.counters, a.counter_elems = buf.data_ptr(), buf.numel()
     else:
         a.counters, a.counter_elems = None, 0

@@ -166,6 +166,56 @@ def test_append_into_strided_cache_views():
 
 
 @pytest.mark.gpu
+def test_decode_and_append_in_one_graph():
+    """The verification step and the cache update captured together in one HIP graph and
+    replayed: each replay attends to the cache as the previous replays left it, appends the
+    accepted rows and advances the lengths in place; an eager loop over the oracle on copies
+    must see the same outputs, caches and lengths after every replay."""
+    from flash_tree_attn_amd import append_accepted_kv, flash_decoding_attention
+    from flash_tree_attn_amd.tree_mask import additive_mask_from_parents, chain_parents
+    from oracle.tree_attn_oracle import tree_attention_oracle
+    g = torch.Generator().manual_seed(21)
+    bsz, hq, hkv, L, D, cap = 2, 8, 2, 8, 128, 512
+    r = lambda *s: torch.randn(*s, generator=g).to(torch.bfloat16).to(DEV)
+    k_cache, v_cache = r(bsz, hkv, cap, D), r(bsz, hkv, cap, D)
+    q, ck, cv = r(bsz, hq, L, D), r(bsz, hkv, L, D), r(bsz, hkv, L, D)
+    lens = torch.tensor([300, 17], dtype=torch.int64, device=DEV)
+    mask = additive_mask_from_parents(chain_parents(L), device=DEV)
+    idx = torch.arange(L, dtype=torch.int32).repeat(bsz, 1).to(DEV)      # a chain: the first n rows are the accepted path
+    n_acc = torch.tensor([3, 5], dtype=torch.int64, device=DEV)
+    out = torch.empty_like(q)
+
+    def step():
+        flash_decoding_attention(q, k_cache, v_cache, ck, cv, mask, lens, kv_group_num=hq // hkv, output=out)
+        append_accepted_kv(k_cache, v_cache, ck, cv, idx, n_acc, lens)
+
+    keep = (k_cache.clone(), v_cache.clone(), lens.clone())
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                                         # warm-up, then put the state back
+        for _ in range(2):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    k_cache.copy_(keep[0]); v_cache.copy_(keep[1]); lens.copy_(keep[2])
+    ref_k, ref_v, ref_lens = (t.clone() for t in keep)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    k_cache.copy_(keep[0]); v_cache.copy_(keep[1]); lens.copy_(keep[2])  # capture does not run the step, but be explicit
+    for rep in range(4):
+        q.copy_(r(bsz, hq, L, D)); ck.copy_(r(bsz, hkv, L, D)); cv.copy_(r(bsz, hkv, L, D))
+        n_acc.copy_(torch.tensor([1 + rep, 5 - rep]))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        ref = tree_attention_oracle(q, ref_k, ref_v, ck, cv, mask, ref_lens, None, hq // hkv)
+        torch.testing.assert_close(out.float(), ref, atol=2e-3, rtol=1e-2)
+        ref_k, ref_v, ref_lens = (t.to(DEV) for t in append_accepted_kv_oracle(ref_k, ref_v, ck, cv, idx, n_acc, ref_lens))
+        assert torch.equal(lens, ref_lens) and torch.equal(k_cache, ref_k) and torch.equal(v_cache, ref_v)
+
+
+@pytest.mark.gpu
 def test_speculative_loop_decode_append_decode():
     """Two verification steps with an append in between equal the oracle run on a cache
     that was extended by hand."""

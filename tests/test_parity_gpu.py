@@ -524,6 +524,39 @@ def test_calls_follow_the_current_stream():
     assert any(k[1] == side.cuda_stream for k in fd._counters)
 
 
+@pytest.mark.parametrize("splits", [1, 3])
+def test_call_under_graph_capture_and_replay(splits):
+    """A serving loop captures its decode step in a HIP graph: the call (one kernel, or stage 1 +
+    stage 2 with the caller's scratch) is captured once and replayed with new data in the same
+    buffers; every replay, with eager work and synchronisations in between, must equal the oracle."""
+    x = make(95, 2, 8, 2, 16, 128, 2048, torch.bfloat16, lens=[2048, 900])
+    out = torch.empty_like(x["q"])
+    mid = torch.empty(2, 8, 4, 16, 128, dtype=torch.float32, device=DEV)
+    lse = torch.empty(2, 8, 4, 16, dtype=torch.float32, device=DEV)
+    call = lambda: run(x, output=out, mid_output=mid, mid_output_lse=lse, _force_splits=splits)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):            # warm-up outside the capture (first-call set-up, remembered signature)
+        for _ in range(3):
+            call()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    check(out, oracle(x), torch.bfloat16)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    g = torch.Generator().manual_seed(7)
+    for rep in range(4):
+        x["q"].copy_(torch.randn(x["q"].shape, generator=g).to(torch.bfloat16))            # eager work between replays
+        x["k_cache"][:, :, :64].copy_(torch.randn(2, 2, 64, 128, generator=g).to(torch.bfloat16))
+        x["kv_seq_len"].copy_(torch.tensor([2048 - 100 * rep, 1 + 300 * rep]))
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        check(out, oracle(x), torch.bfloat16)
+
+
 def test_paged_argument_errors():
     x = make(82, 2, 4, 2, 8, 128, 128, torch.float16, [128, 5])
     kp, vp, tables = to_pages(x, 32, seed=1)
