@@ -35,8 +35,9 @@ def parse():
     ap.add_argument("--config", default="cfg3_gqa_8b_bf16", help="workload name (flash_tree_attn_amd.synthetic.CONFIGS)")
     ap.add_argument("--kv-sets", type=int, default=0, help="independent KV caches to rotate over (0 = enough for >1 GiB)")
     ap.add_argument("--splits", type=int, default=0, help="pin the split count (0 = heuristic)")
-    ap.add_argument("--kernel", default="auto", choices=["auto", "mfma", "shuffle"],
-                    help="pin the stage-1 kernel (auto = the plan's choice); for comparing the two on one workload")
+    ap.add_argument("--kernel", default="auto", choices=["auto", "mfma", "mfma_wide", "shuffle"],
+                    help="pin the stage-1 kernel (auto = the plan's choice); for comparing them on one workload. mfma_wide = the "
+                         "MFMA kernel with 64-row waves and the hand-scheduled half-tile loop (256-row units, contiguous caches)")
     ap.add_argument("--op", default="decode", choices=["decode", "append_kv"],
                     help="decode = the tree-attention call (the headline); append_kv = the accepted-path KV append that follows it")
     ap.add_argument("--accept", type=int, default=8, help="accepted tree rows per sequence for --op append_kv")
@@ -44,9 +45,6 @@ def parse():
                     help="run on paged caches: pages of PAGE positions (16/32/64/128), shuffled in one pool, with a block table")
     ap.add_argument("--packed-mask", action="store_true", help="pass the tree mask as packed bit words instead of float32")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--machine-probe", action="store_true",
-                    help="only run the machine characterisation probes (dense MFMA rate and clock, matrix/vector overlap, "
-                         "streaming rate of the HBM -> LDS load pattern) and print them as one JSON line")
     ap.add_argument("--reference-sweep", action="store_true",
                     help="only run the sweep of the reference's own benchmark (flash_tree_attn.py:442-487: bsz 2, 32 MHA heads, "
                          "D 128, fp16, q_len 16..128 x context 64..256, K/V passed as slices of one buffer) through the drop-in "
@@ -103,44 +101,6 @@ def cpu_baseline(cfg, x, budget_s):
                   f"{t * 1e6 / nseq * cfg.bsz:.0f} us/call extrapolated to the full batch, os.cpu_count()={os.cpu_count()}",
         "us_per_call_extrapolated": t * 1e6 / nseq * cfg.bsz,
     }
-
-
-def machine_probe():
-    """Runs the probes of libfta_probe.so (flash_tree_attn_amd/csrc/machine_probe.hip)."""
-    import ctypes as C
-    from flash_tree_attn_amd.build import PROBE_LIB_PATH
-    if not os.path.exists(PROBE_LIB_PATH):
-        raise ImportError(f"{PROBE_LIB_PATH} is missing: build it with `python -m flash_tree_attn_amd.build`")
-    lib = C.CDLL(PROBE_LIB_PATH)
-    lib.fta_machine_probe.restype = C.c_int
-    lib.fta_machine_probe.argtypes = [C.c_int, C.c_int, C.POINTER(C.c_double)]
-    names = ["mfma_1_wave_per_simd", "mfma_2_waves_per_simd", "fma_1_wave_per_simd", "roles_mfma_wave_plus_fma_wave",
-             "mixed_both_waves_interleave", "stream_hbm_to_lds", "stream_hbm_to_registers"]
-    res = {}
-    for which, name in enumerate(names):
-        out = (C.c_double * 3)()
-        # a first call settles the clocks, the second is reported
-        for _ in range(2):
-            if lib.fta_machine_probe(which, 20 if which < 5 else 10, out) != 0:
-                raise RuntimeError(f"probe {name} failed")
-        ms, mhz, work = out[0], out[1], out[2]
-        entry = {"ms": round(ms, 4), "shader_clock_mhz": round(mhz)}
-        if which in (0, 1, 3, 4):
-            entry["mfma_tflops"] = round(work / (ms * 1e-3) / 1e12, 1)
-        elif which == 2:
-            entry["fma_lane_ops_per_s"] = work / (ms * 1e-3)
-        else:
-            entry["gbs"] = round(work / (ms * 1e-3) / 1e9, 1)
-        res[name] = entry
-    t = lambda n: res[n]["ms"]
-    res["overlap"] = {
-        "roles_over_sum": round(t("roles_mfma_wave_plus_fma_wave") / (t("mfma_1_wave_per_simd") + t("fma_1_wave_per_simd")), 3),
-        "mixed_over_sum": round(t("mixed_both_waves_interleave") / (t("mfma_2_waves_per_simd") + 2 * t("fma_1_wave_per_simd")), 3),
-        "note": "time of the combination over the sum of its parts run alone: 1.0 = matrix and vector time add up, "
-                "max(a,b)/(a+b) = full overlap. 'roles' = one MFMA wave next to one FMA wave on every SIMD; 'mixed' = both "
-                "waves of every SIMD interleave 1 MFMA + 8 FMA (parts: the 2-wave MFMA probe and twice the 1-wave FMA probe)",
-    }
-    print(json.dumps({"machine_probe": res}))
 
 
 def reference_sweep(dev):
@@ -263,8 +223,6 @@ def main():
     cfg = CONFIGS[args.config]
     dev = "cuda:0"
     torch.cuda.set_device(0)
-    if args.machine_probe:
-        return machine_probe()
     if args.reference_sweep:
         return reference_sweep(dev)
     if args.copy_calibration:
@@ -309,7 +267,7 @@ def main():
                 x["k_cache_paged"], x["v_cache_paged"], x["tables"] = kc, vc, tables
         calls.append(prepare(x["q"], kc, vc, x["current_k"], x["current_v"], mask_arg, x["kv_seq_len"], cfg.block_size,
                              None, None, None, None, x["sm_scale"], cfg.kv_group_num, _force_splits=args.splits,
-                             _force_kernel={"auto": -1, "mfma": _lib.KERNEL_MFMA, "shuffle": _lib.KERNEL_SHUFFLE}[args.kernel],
+                             _force_kernel={"auto": -1, "mfma": _lib.KERNEL_MFMA, "mfma_wide": _lib.KERNEL_MFMA_WIDE, "shuffle": _lib.KERNEL_SHUFFLE}[args.kernel],
                              block_tables=tables))
     if args.paged:   # the contiguous copies are no longer needed, except set 0 for the self-check
         x["k_caches"], x["v_caches"] = x["k_caches"][:1], x["v_caches"][:1]
@@ -345,7 +303,14 @@ def main():
         torch.cuda.synchronize()
     for i in range(args.warmup):
         calls[i % kv_sets].run()
-    ms = timed("run", args.steps)
+    # the timed region: exactly --steps calls, event-timed in batches of 25 (the last may be shorter). The headline is
+    # the median batch, so that one disturbed batch (a clock dip, another tenant of the host) does not move it; the
+    # mean over all steps is reported beside it.
+    sizes = [25] * (args.steps // 25) + ([args.steps % 25] if args.steps % 25 else [])
+    batch_ms = [timed("run", n) for n in sizes]
+    ms_mean = sum(b * n for b, n in zip(batch_ms, sizes)) / args.steps
+    batch_sorted = sorted(batch_ms)
+    ms = batch_sorted[len(batch_sorted) // 2]
     single_launch = bool(plan.single_launch)   # the merge runs inside the stage-1 kernel
     ms_two = timed("run_two_launches", args.steps) if single_launch else ms
     ms_stage1_alone = timed("run_stage1", args.steps)
@@ -353,29 +318,16 @@ def main():
     # the dominant kernel as launched in the timed region: with the merge inside, the call IS that kernel
     ms_stage1 = ms if single_launch else ms_stage1_alone
 
-    # spread of the whole-call time: 20 separately timed batches of 25 calls
-    batch_us = sorted(timed("run", 25) * 1e3 for _ in range(20))
-
-    # shader clock the card holds under the stage-1 kernel (measurement hook of the library)
-    clock_mhz = None
-    if plan.kernel == _lib.KERNEL_MFMA:
-        lib = _lib.load()
-        clk = torch.zeros(2, dtype=torch.int64, device=dev)
-        lib.fta_debug_clock_buffer(clk.data_ptr())
-        for i in range(8):
-            calls[i % kv_sets].run_stage1()
-        torch.cuda.synchronize()
-        lib.fta_debug_clock_buffer(None)
-        cyc, ticks = (int(v) for v in clk.tolist())
-        clock_mhz = round(cyc / (ticks / 100.0)) if ticks > 0 else None
-
     gbs = nbytes / (ms * 1e-3) / 1e9
     gbs_s1 = nbytes / (ms_stage1 * 1e-3) / 1e9
     result = {
         "metric": "tree-attn us/call + achieved HBM GB/s (% peak), 8B GQA q_len=64 @8K ctx",
         "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "settle_ms": args.settle_ms, "ms_per_step": ms, "us_per_call": ms * 1e3,
-        "us_per_call_batches": {"median": round(batch_us[10], 2), "min": round(batch_us[0], 2), "max": round(batch_us[-1], 2), "batches": 20, "calls_per_batch": 25}, "pct_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
+        "ms_per_step_is": "median of the event-timed batches of the --steps calls", "ms_per_step_mean": ms_mean,
+        "us_per_call_batches": {"median": round(ms * 1e3, 2), "min": round(batch_sorted[0] * 1e3, 2),
+                                "max": round(batch_sorted[-1] * 1e3, 2), "batches": len(sizes), "calls_per_batch": 25},
+        "pct_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}[cfg.dtype],
         "data": "synthetic (seed 0, N(0,1) q/k/v, random tree mask), inputs resident in HBM",
@@ -383,17 +335,18 @@ def main():
                    "head_dim": cfg.head_dim, "q_len": cfg.q_len, "cache_len": cfg.cache_len, "lengths": cfg.lengths,
                    "block_size": cfg.block_size, "mask": "packed u64" if args.packed_mask else "additive f32",
                    "kv_layout": f"paged, {args.paged} positions per page, shuffled pool" if args.paged else "contiguous per sequence", "kv_sets_rotated": kv_sets, "num_splits": plan.num_splits,
-                   "chunk": plan.chunk, "stage1_kernel": "mfma" if plan.kernel == _lib.KERNEL_MFMA else "shuffle",
+                   "chunk": plan.chunk, "stage1_kernel": ("mfma_wide" if plan.mfma_loop else "mfma") if plan.kernel == _lib.KERNEL_MFMA else "shuffle",
                    "stage1_workgroups": plan.num_workgroups, "algorithmic_bytes": nbytes, "flops": nflops},
         "tflops": nflops / (ms * 1e-3) / 1e12,
         "roofline": {"bound": "hbm", "kernel": "stage1", "achieved": round(gbs_s1, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(gbs_s1 / HBM_PEAK_GBS, 4), "traffic": traffic_from_profiles(cfg.name),
+                     "traffic_source": None if traffic_from_profiles(cfg.name) is None else f"profiles/stage1_{cfg.name}_pmc.txt (rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE of an "
+                                       "earlier run of this command, scaled by a plain copy; not measured in this run)",
                      "us_per_launch": ms_stage1 * 1e3, "single_launch": single_launch,
                      "two_launch_call_us": ms_two * 1e3, "stage1_without_merge_us": ms_stage1_alone * 1e3,
                      "stage2_us_per_launch": ms_stage2 * 1e3,
                      "mfma_tflops": nflops / (ms_stage1 * 1e-3) / 1e12,
-                     "mfma_frac_of_dense_peak": round(nflops / (ms_stage1 * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4),
-                     "shader_clock_mhz_under_kernel": clock_mhz},
+                     "mfma_frac_of_dense_peak": round(nflops / (ms_stage1 * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4)},
     }
     # context for the datasheet peak: what a plain device copy of 1 GiB streams on this box (read + write bytes)
     src = torch.empty(1 << 29, dtype=torch.bfloat16, device=dev).normal_()

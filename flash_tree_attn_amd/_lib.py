@@ -7,15 +7,15 @@ import os
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libfta.so")
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 FTA_F32, FTA_F16, FTA_BF16 = 0, 1, 2
 FTA_I32, FTA_I64 = 0, 1
 MASK_ADDITIVE_F32, MASK_PACKED_U64 = 0, 1
-KERNEL_SHUFFLE, KERNEL_MFMA = 0, 1
+KERNEL_SHUFFLE, KERNEL_MFMA, KERNEL_MFMA_WIDE = 0, 1, 2
 
 EXPORTED_SYMBOLS = (
     "fta_abi_version", "fta_strerror", "fta_validate", "fta_plan", "fta_decode", "fta_decode_stage1",
-    "fta_decode_stage2", "fta_device_cus", "fta_append_kv", "fta_debug_clock_buffer",
+    "fta_decode_stage2", "fta_device_cus", "fta_append_kv",
 )
 
 # status -> Python exception class
@@ -57,7 +57,7 @@ class FtaPlanOut(C.Structure):
     _fields_ = [
         ("kernel", C.c_int32), ("num_splits", C.c_int32), ("chunk", C.c_int32), ("rows_per_group", C.c_int32),
         ("rows_per_wg", C.c_int32), ("row_blocks", C.c_int32), ("num_workgroups", C.c_int32), ("counter_elems", C.c_int32),
-        ("single_launch", C.c_int32), ("reserved", C.c_int32),
+        ("single_launch", C.c_int32), ("mfma_loop", C.c_int32),
         ("mid_o_elems", C.c_int64), ("mid_lse_elems", C.c_int64),
     ]
 
@@ -96,8 +96,6 @@ def load() -> C.CDLL:
         fn.restype = C.c_int
         fn.argtypes = [C.POINTER(FtaArgs), C.c_void_p]
     lib.fta_device_cus.restype = C.c_int
-    lib.fta_debug_clock_buffer.restype = C.c_int
-    lib.fta_debug_clock_buffer.argtypes = [C.c_void_p]
     lib.fta_append_kv.restype = C.c_int
     lib.fta_append_kv.argtypes = [C.POINTER(FtaAppendArgs), C.c_void_p]
     if lib.fta_abi_version() != ABI_VERSION:

@@ -14,9 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 LIB_PATH = os.path.join(HERE, "libfta.so")
-PROBE_LIB_PATH = os.path.join(HERE, "libfta_probe.so")   # machine characterisation kernels for `bench.py --machine-probe`
-PROBE_SOURCES = ["machine_probe.hip"]
-SOURCES = ["fta_host.cpp", "stage1_shuffle.hip", "stage1_mfma.hip", "stage2_merge.hip", "append_kv.hip"]
+SOURCES = ["fta_host.cpp", "stage1_shuffle.hip", "stage1_mfma.hip", "stage1_mfma_wide.hip", "stage2_merge.hip", "append_kv.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
@@ -26,7 +24,7 @@ FLAGS = [
     # the kernels use -inf as the "masked" logit.
     "-fno-honor-nans",
     "-I", INCLUDE, "-I", CSRC,
-]
+] + os.environ.get("FTA_EXTRA_FLAGS", "").split()
 
 
 def _compile(src: str) -> str:
@@ -51,16 +49,27 @@ def _link(objs, path: str) -> None:
         raise RuntimeError(f"link failed:\n{res.stderr}")
 
 
+def _generate() -> None:
+    """Rewrites csrc/wide_loop_asm.inc from its generator (deterministic; the file is committed)."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("gen_wide_loop", os.path.join(CSRC, "gen_wide_loop.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    text = mod.render()
+    path = os.path.join(CSRC, "wide_loop_asm.inc")
+    if not os.path.exists(path) or open(path).read() != text:
+        with open(path, "w") as f:
+            f.write(text)
+
+
 def build(verbose: bool = True) -> str:
-    """Compiles every HIP source: the product library and the machine-probe library."""
-    all_sources = SOURCES + PROBE_SOURCES
-    with ThreadPoolExecutor(max_workers=min(6, len(all_sources))) as pool:
-        objs = list(pool.map(_compile, all_sources))
-    _link(objs[:len(SOURCES)], LIB_PATH)
-    _link(objs[len(SOURCES):], PROBE_LIB_PATH)
+    """Compiles every HIP source of the library and links it."""
+    _generate()
+    with ThreadPoolExecutor(max_workers=min(6, len(SOURCES))) as pool:
+        objs = list(pool.map(_compile, SOURCES))
+    _link(objs, LIB_PATH)
     if verbose:
         print(f"built {LIB_PATH}")
-        print(f"built {PROBE_LIB_PATH}")
     return LIB_PATH
 
 

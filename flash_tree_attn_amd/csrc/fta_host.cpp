@@ -11,14 +11,26 @@
 
 namespace fta {
 
+const EnvKnobs& env_knobs() {
+  static const EnvKnobs knobs = [] {
+    EnvKnobs k{};
+    if (const char* e = std::getenv("FTA_ROWS_PER_WG")) k.rows_128 = std::atoi(e) == 128;
+    if (const char* e = std::getenv("FTA_FORCE_SPLITS")) k.force_splits = std::max(0, std::atoi(e));
+    k.tree_tile_weight = -1;
+    if (const char* e = std::getenv("FTA_TREE_TILE_WEIGHT")) k.tree_tile_weight = std::max(0, std::atoi(e));
+    if (const char* e = std::getenv("FTA_WIDE_LOOP")) k.wide_loop = e[0] == '1';
+    return k;
+  }();
+  return knobs;
+}
+
 // Query rows one MFMA workgroup holds: 256 (8 waves x 32 rows, two waves per SIMD, one
 // workgroup per CU: the K/V rings take most of the LDS) when the unit has more than 128
 // rows, else 128 (4 waves, short rings, two workgroups per CU). FTA_ROWS_PER_WG=128
 // forces the 4-wave variant (tuning only). head_dim 256 only exists as the 4-wave variant:
 // its tiles are twice as large, two K and two V stages fill the LDS of a CU.
 int mfma_rows_per_wg(int rows, int head_dim) {
-  if (const char* env = std::getenv("FTA_ROWS_PER_WG"))
-    if (std::atoi(env) == 128) return 128;
+  if (env_knobs().rows_128) return 128;
   return rows > 128 && head_dim <= 128 ? 256 : 128;
 }
 
@@ -62,7 +74,9 @@ int validate(const fta_args& a) {
     return FTA_ERR_SHAPE;
   if (a.num_q_heads % a.num_kv_heads != 0) return FTA_ERR_SHAPE;
   if (a.cur_heads != a.num_kv_heads && a.cur_heads != a.num_q_heads) return FTA_ERR_SHAPE;
-  if (a.force_kernel < -1 || a.force_kernel > FTA_KERNEL_MFMA) return FTA_ERR_UNSUPPORTED;
+  if (a.force_kernel < -1 || a.force_kernel > FTA_KERNEL_MFMA_WIDE) return FTA_ERR_UNSUPPORTED;
+  // Paged caches with no capacity have no table entry to look up (the kernels clamp positions to cache_len - 1).
+  if (a.block_table && a.cache_len == 0) return FTA_ERR_SHAPE;
 
   // Rows are moved with 128-bit accesses: every row start must be 16-byte aligned.
   const int vec = 16 / esize(a.dtype);
@@ -89,10 +103,16 @@ int plan(const fta_args& a, int num_cus, fta_plan_out* out) {
 
   int kernel = mfma_eligible(a) ? FTA_KERNEL_MFMA : FTA_KERNEL_SHUFFLE;
   if (a.force_kernel >= 0) {
-    if (a.force_kernel == FTA_KERNEL_MFMA && !mfma_eligible(a)) return FTA_ERR_UNSUPPORTED;
-    kernel = a.force_kernel;
+    if (a.force_kernel != FTA_KERNEL_SHUFFLE && !mfma_eligible(a)) return FTA_ERR_UNSUPPORTED;
+    kernel = a.force_kernel == FTA_KERNEL_SHUFFLE ? FTA_KERNEL_SHUFFLE : FTA_KERNEL_MFMA;
   }
   const int rows_per_wg = kernel == FTA_KERNEL_MFMA ? mfma_rows_per_wg(rows, a.head_dim) : 16;
+  // The 64-row-wave loop serves 256-row workgroups on contiguous caches, head_dim 64 / 128. It is
+  // opt-in (force_kernel or FTA_WIDE_LOOP=1): at the headline shape it measures level with the
+  // 8-wave loop, ahead of it on long chunks and behind it on short ones.
+  const bool wide_ok = kernel == FTA_KERNEL_MFMA && rows_per_wg == 256 && !a.block_table && a.head_dim <= 128;
+  if (a.force_kernel == FTA_KERNEL_MFMA_WIDE && !wide_ok) return FTA_ERR_UNSUPPORTED;
+  const bool wide = wide_ok && (a.force_kernel == FTA_KERNEL_MFMA_WIDE || (a.force_kernel < 0 && env_knobs().wide_loop));
   const int row_blocks = static_cast<int>(cdiv(rows, rows_per_wg));
   // Workgroups one CU holds at a time (LDS- and register-bound, see the kernels): the
   // 128-row MFMA variant is built to share a CU with a second workgroup.
@@ -151,10 +171,7 @@ int plan(const fta_args& a, int num_cus, fta_plan_out* out) {
       if (cost_of[cand] <= cost_of[chosen] * 1.10) splits = cand;
   }
   if (a.force_splits > 0) splits = a.force_splits;
-  if (const char* env = std::getenv("FTA_FORCE_SPLITS")) {
-    const int v = std::atoi(env);
-    if (v > 0) splits = v;
-  }
+  if (env_knobs().force_splits > 0) splits = env_knobs().force_splits;
   // Never more splits than blocks of the reference granularity, so that a scratch
   // buffer sized like the reference's (flash_tree_attn.py:274-281) always fits.
   splits = std::min<int64_t>(splits, std::max<int64_t>(1, cdiv(t_cap, gran)));
@@ -162,8 +179,7 @@ int plan(const fta_args& a, int num_cus, fta_plan_out* out) {
   // latency-bound step worth about three cache tiles per tree tile): count it as extra
   // keys when cutting chunks, so that the last split of a full-length sequence gets a
   // correspondingly shorter cache range.
-  int64_t tree_weight = 3;
-  if (const char* env = std::getenv("FTA_TREE_TILE_WEIGHT")) tree_weight = std::max(0, std::atoi(env));
+  const int64_t tree_weight = env_knobs().tree_tile_weight >= 0 ? env_knobs().tree_tile_weight : 3;
   const int64_t tree_keys = splits > 1 ? tree_weight * kKeyTile * cdiv(a.q_len, kKeyTile) : 0;
   int64_t chunk = cdiv(cdiv(std::max<int64_t>(t_cap, 1) + tree_keys, splits), gran) * gran;
   if ((splits - 1) * chunk >= std::max<int64_t>(t_cap, 1)) chunk = cdiv(cdiv(std::max<int64_t>(t_cap, 1), splits), gran) * gran;
@@ -176,7 +192,7 @@ int plan(const fta_args& a, int num_cus, fta_plan_out* out) {
   out->rows_per_wg = rows_per_wg;
   out->row_blocks = row_blocks;
   out->num_workgroups = static_cast<int32_t>(work_items * splits);
-  out->reserved = 0;
+  out->mfma_loop = wide ? 1 : 0;
   out->counter_elems = (splits > 1 && kernel == FTA_KERNEL_MFMA && work_items <= 0x7fffffff) ? static_cast<int32_t>(work_items) : 0;
   // Merging inside stage 1 saves the second launch, but the last workgroup of a sequence
   // merges alone: that pays with two splits and one round of workgroups (short launches,
@@ -192,16 +208,7 @@ int plan(const fta_args& a, int num_cus, fta_plan_out* out) {
 
 extern "C" {
 
-namespace {
-long long* g_clock_out = nullptr;   // see fta_debug_clock_buffer
-}
-
 int fta_abi_version(void) { return FTA_ABI_VERSION; }
-
-int fta_debug_clock_buffer(void* two_int64_on_device) {
-  g_clock_out = static_cast<long long*>(two_int64_on_device);
-  return FTA_OK;
-}
 
 const char* fta_strerror(int status) {
   switch (status) {
@@ -279,9 +286,9 @@ int decode_impl(const fta_args* args, void* hip_stream, int stages) {
   p.mask = a.mask; p.lens = a.kv_seq_len; p.out = a.out; p.mid_o = a.mid_o; p.mid_lse = a.mid_lse;
   p.counters = fused ? a.counters : nullptr;
   p.block_table = a.block_table;
-  p.clock_out = g_clock_out;
   p.table_stride = a.block_table_stride;
   p.page_shift = a.page_size == 16 ? 4 : a.page_size == 32 ? 5 : a.page_size == 64 ? 6 : 7;
+  p.wide_loop = pl.mfma_loop;
   p.bsz = a.bsz; p.num_q_heads = a.num_q_heads; p.q_len = a.q_len; p.cache_len = a.cache_len;
   p.chunk = pl.chunk; p.num_splits = pl.num_splits;
   p.heads_per_unit = pl.rows_per_group / a.q_len;

@@ -25,7 +25,6 @@ struct KernelParams {
   float* mid_o;
   float* mid_lse;
   const int32_t* block_table;  // null = contiguous caches; else page index per (sequence, position / page size)
-  long long* clock_out;   // measurement hook: {shader cycles, 100 MHz ticks} of workgroup 0, or null
   int32_t* counters;      // one per (sequence, unit, row block) when the merge runs inside stage 1, else null
 
   int32_t bsz;
@@ -45,6 +44,7 @@ struct KernelParams {
   int32_t mask_vec4;      // every (float) mask row starts 16-byte aligned
   int32_t mask_packed;    // mask holds one bit per (row, tree key): set = attend
   int32_t page_shift;     // log2(page size) when block_table is set
+  int32_t wide_loop;      // 256-row workgroups: 4 waves x 64 rows with the half-tile loop instead of 8 waves x 32 rows
   float scale_log2;       // sm_scale * log2(e)
 
   int64_t q_stride[3];
@@ -62,9 +62,20 @@ struct KernelParams {
 // Launchers implemented in the .hip files. Each returns a fta_status.
 int launch_stage1_shuffle(const KernelParams& p, int dtype, int head_dim, void* stream);
 int launch_stage1_mfma(const KernelParams& p, int dtype, int head_dim, void* stream);
+int launch_stage1_mfma_wide(const KernelParams& p, int dtype, int head_dim, void* stream);   // 256-row workgroups of 64-row waves
 int launch_stage2_merge(const KernelParams& p, int dtype, int head_dim, void* stream);
 
 // Rows one MFMA workgroup holds for a unit of `rows` query rows (host + device agree on it).
 int mfma_rows_per_wg(int rows, int head_dim);
+
+// Tuning knobs from the environment, read once per process (comparison runs and tests only):
+// FTA_ROWS_PER_WG=128, FTA_FORCE_SPLITS=n, FTA_TREE_TILE_WEIGHT=n, FTA_WIDE_LOOP=1.
+struct EnvKnobs {
+  bool rows_128;
+  int force_splits;      // 0 = none
+  int tree_tile_weight;  // < 0 = default
+  bool wide_loop;
+};
+const EnvKnobs& env_knobs();
 
 }  // namespace fta

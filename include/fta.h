@@ -20,7 +20,7 @@
 extern "C" {
 #endif
 
-#define FTA_ABI_VERSION 2
+#define FTA_ABI_VERSION 3
 
 typedef enum fta_status {
   FTA_OK = 0,
@@ -50,7 +50,10 @@ typedef enum fta_mask_kind {
 /* Which stage-1 kernel a plan selects. */
 typedef enum fta_kernel {
   FTA_KERNEL_SHUFFLE = 0,  /* wavefront-shuffle reductions: any dtype / head_dim / q_len / sign of sm_scale */
-  FTA_KERNEL_MFMA = 1      /* MFMA tiles: f16/bf16, head_dim 64/128/256, sm_scale > 0; any number of rows */
+  FTA_KERNEL_MFMA = 1,     /* MFMA tiles: f16/bf16, head_dim 64/128/256, sm_scale > 0; any number of rows */
+  FTA_KERNEL_MFMA_WIDE = 2 /* only as fta_args.force_kernel: the MFMA kernel with 64 query rows per wave and the
+                              hand-scheduled half-tile loop, for units of more than 128 rows on contiguous caches,
+                              head_dim 64/128. A plan reports it as FTA_KERNEL_MFMA with mfma_loop = 1. */
 } fta_kernel;
 
 /*
@@ -113,7 +116,7 @@ typedef struct fta_args {
   int32_t dtype;            /* fta_dtype of q/k/v/cur/out */
   int32_t len_dtype;        /* fta_len_dtype of kv_seq_len */
   int32_t force_splits;     /* 0 = heuristic; >0 pins the split count (tuning, tests) */
-  int32_t force_kernel;     /* -1 = heuristic; else an fta_kernel */
+  int32_t force_kernel;     /* -1 = heuristic; else an fta_kernel (FTA_ERR_UNSUPPORTED where that kernel cannot run the call) */
   int32_t counter_elems;    /* int32 elements behind `counters`, 0 when it is NULL */
   int32_t mask_kind;        /* fta_mask_kind of `mask` */
   int32_t page_size;        /* positions per page, one of 16, 32, 64, 128; ignored without block_table */
@@ -144,7 +147,7 @@ typedef struct fta_plan_out {
   int32_t single_launch;  /* 1 where the single-launch path is expected to be the faster one (two splits, one
                              round of workgroups: the last workgroup of a sequence merges alone, which does
                              not pay for more) */
-  int32_t reserved;
+  int32_t mfma_loop;      /* MFMA kernel, 256-row workgroups: 0 = 8 waves x 32 rows, 1 = 4 waves x 64 rows (half-tile loop) */
   int64_t mid_o_elems;    /* float32 elements a dense mid_o for this plan needs */
   int64_t mid_lse_elems;
 } fta_plan_out;
@@ -227,12 +230,6 @@ typedef struct fta_append_args {
 
 /* Validates, then launches on `hip_stream`. Asynchronous; allocates nothing. */
 int fta_append_kv(const fta_append_args* args, void* hip_stream);
-
-/* Measurement hook (no counterpart in the reference): with a device buffer of two int64 set, workgroup 0
- * of every later stage-1 MFMA launch stores there the shader-clock cycles and the 100 MHz reference ticks
- * it ran for; their ratio is the clock the card held under the kernel (bench.py reports it). NULL (the
- * default) switches it off. Process-wide; not meant for concurrent use. */
-int fta_debug_clock_buffer(void* two_int64_on_device);
 
 /* Number of compute units of the current HIP device, or a negative fta_status. */
 int fta_device_cus(void);

@@ -216,6 +216,34 @@ def test_plan_overrides(fta_lib):
     assert st == -9
 
 
+def test_plan_of_the_64_row_wave_loop(fta_lib):
+    """The hand-scheduled loop is a choice of the caller: units of 256 rows on contiguous caches,
+    head_dim 64 or 128. Asked for anywhere else it is refused, never silently replaced."""
+    wide = dict(num_q_heads=32, num_kv_heads=8, cur_heads=8, q_len=64, force_kernel=_lib.KERNEL_MFMA_WIDE)
+    st, pl = plan(fta_lib, base_args(**wide))
+    assert st == 0 and pl.kernel == _lib.KERNEL_MFMA and pl.rows_per_wg == 256 and pl.mfma_loop == 1
+    st, pl = plan(fta_lib, base_args(**{**wide, "force_kernel": _lib.KERNEL_MFMA}))
+    assert st == 0 and pl.rows_per_wg == 256 and pl.mfma_loop == 0
+    if not os.environ.get("FTA_WIDE_LOOP"):
+        st, pl = plan(fta_lib, base_args(**{**wide, "force_kernel": -1}))
+        assert st == 0 and pl.mfma_loop == 0
+    assert plan(fta_lib, base_args(**{**wide, "q_len": 8}))[0] == -9              # 32-row units
+    assert plan(fta_lib, base_args(**{**wide, "head_dim": 256}))[0] == -9
+    assert plan(fta_lib, base_args(**{**wide, "dtype": _lib.FTA_F32}))[0] == -9
+    a = base_args(**wide)                                                         # paged caches: 64 pages of 128 positions per sequence
+    table = (C.c_int32 * (8 * 64))()
+    a.block_table, a.block_table_stride, a.page_size = C.cast(table, C.c_void_p), 64, 128
+    a.k_stride[0] = a.v_stride[0] = 8 * 128 * 128
+    a.k_stride[1] = a.v_stride[1] = 128 * 128
+    assert fta_lib.fta_validate(C.byref(a)) == 0 and plan(fta_lib, a)[0] == -9
+    a.force_kernel = -1
+    st, pl = plan(fta_lib, a)
+    assert st == 0 and pl.rows_per_wg == 256 and pl.mfma_loop == 0
+    # a paged cache of no positions has no pages to name: rejected as a shape error
+    a.cache_len = a.v_cache_len = 0
+    assert fta_lib.fta_validate(C.byref(a)) == -7
+
+
 def test_python_wrapper_rejects_cpu_tensors():
     """No CPU fallback: the product path refuses CPU tensors outright."""
     import torch

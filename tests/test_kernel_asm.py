@@ -1,103 +1,162 @@
-"""Static check of the compiled stage-1 MFMA kernels (device assembly, no GPU needed).
+"""Static checks of the stage-1 MFMA kernels: the device assembly hipcc emits for them and the
+hand-scheduled loop's generator (no GPU needed).
 
-The kernel loads its Q rows with inline-assembly global loads that the compiler's wait
-insertion does not see, and waits for them by hand. Between such a load and the wait the
-destination registers hold stale values and receive the data at an unknown moment: if the
-compiler copied, spilled or reused them there, the late data would land in whatever lives
-in them by then (an address, say). This test reads the assembly hipcc emits for every
-instantiation and asserts that nothing touches those registers inside the window."""
+The kernels wait for their HBM -> LDS loads by hand (`s_waitcnt vmcnt(n)` with n counted from
+the loads the code itself issued). That is only sound for loads whose destination is LDS: a
+hand-issued load into REGISTERS is invisible to the compiler's wait insertion, and until the
+hand-written wait the compiler may copy, spill or reuse the destination. The kernels therefore
+contain no such load, and the first test keeps it that way.
+
+The 64-row-wave loop is one inline-assembly statement over fixed physical registers. The
+compiler keeps its own values in every register the statement does not declare, so the
+statement's operand and clobber lists must name every register its text touches: the
+generator checks that when it renders, and the tests here check the checker."""
+import importlib.util
 import os
 import re
 import subprocess
 import tempfile
+from concurrent.futures import ThreadPoolExecutor
 
 import pytest
 
 from flash_tree_attn_amd import build as fta_build
 
-SRC = os.path.join(fta_build.CSRC, "stage1_mfma.hip")
-REG = re.compile(r"\bv(\d+)\b|\bv\[(\d+):(\d+)\]")
+UNITS = ["stage1_mfma.hip", "stage1_mfma_wide.hip"]
 
 
-def regs_of(text):
-    out = set()
-    for m in REG.finditer(text):
-        if m.group(1) is not None:
-            out.add(int(m.group(1)))
-        else:
-            out.update(range(int(m.group(2)), int(m.group(3)) + 1))
-    return out
+def _generator():
+    spec = importlib.util.spec_from_file_location("gen_wide_loop", os.path.join(fta_build.CSRC, "gen_wide_loop.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
 
 
 @pytest.fixture(scope="module")
 def kernels():
+    """name -> (instruction lines, metadata dict) of every stage1_mfma_kernel instantiation."""
     if not os.path.exists(fta_build.HIPCC):
         pytest.skip("hipcc not available")
     with tempfile.TemporaryDirectory() as tmp:
-        out = os.path.join(tmp, "stage1_mfma.s")
-        cmd = [fta_build.HIPCC, *fta_build.FLAGS, "--cuda-device-only", "-S", "-x", "hip", SRC, "-o", out]
-        subprocess.run(cmd, check=True, capture_output=True)
-        text = open(out).read()
-    bodies = {}
-    for m in re.finditer(r"^(_ZN3fta\S*stage1_mfma_kernel[^:\s]*):[^\n]*\n(.*?)^\.Lfunc_end", text, flags=re.S | re.M):
-        lines = [l.split(";")[0].strip() if not l.strip().startswith(";;#ASM") else l.strip() for l in m.group(2).split("\n")]
-        bodies[m.group(1)] = [l for l in lines if l and not l.startswith(".") and not l.endswith(":")]
-    assert len(bodies) >= 12, "expected every dtype x head_dim x variant x paged instantiation"
-    return bodies
+        def compile_unit(src):
+            out = os.path.join(tmp, src + ".s")
+            cmd = [fta_build.HIPCC, *fta_build.FLAGS, "--cuda-device-only", "-S", "-x", "hip", os.path.join(fta_build.CSRC, src), "-o", out]
+            subprocess.run(cmd, check=True, capture_output=True)
+            return open(out).read()
+        with ThreadPoolExecutor(max_workers=2) as pool:
+            texts = list(pool.map(compile_unit, UNITS))
+    found = {}
+    for text in texts:
+        meta = {}
+        for entry in text.split("\n  - .agpr_count:")[1:]:
+            field = lambda key: re.search(rf"^\s+\.{key}:\s+(\S+)", entry, flags=re.M).group(1)
+            meta[field("name")] = {"agpr": int(entry.split()[0]), "scratch": int(field("private_segment_fixed_size")), "vgpr": int(field("vgpr_count"))}
+        for m in re.finditer(r"^(_ZN3fta\S*stage1_mfma_kernel[^:\s]*):[^\n]*\n(.*?)^\.Lfunc_end", text, flags=re.S | re.M):
+            lines = [l.strip() if l.strip().startswith(";;#ASM") else l.split(";")[0].strip() for l in m.group(2).split("\n")]
+            found[m.group(1)] = ([l for l in lines if l and not l.startswith(".") and not l.endswith(":")], meta[m.group(1)])
+    # 2 dtypes x paged/contiguous x (pipelined D 128, 64 + plain D 128, 64, 256) + 2 dtypes x wide D 128, 64
+    assert len(found) == 2 * 2 * 5 + 2 * 2, sorted(found)
+    return found
 
 
-def test_untracked_q_loads_are_not_touched_before_their_wait(kernels):
-    for name, ins in kernels.items():
-        # inline-assembly register loads without a cache-scope modifier = the Q rows
-        in_asm, q_loads = False, []
-        for i, l in enumerate(ins):
-            if l.startswith(";;#ASMSTART"):
-                in_asm = True
-            elif l.startswith(";;#ASMEND"):
-                in_asm = False
-            elif in_asm and l.startswith("global_load_dwordx4") and "sc1" not in l:
-                q_loads.append(i)
-        # the Q loads are the first group of such loads; the merge code (sc1) is excluded above, and
-        # nothing else in the kernel uses an untracked register load
-        first = q_loads[0]
-        group = [i for i in q_loads if i - first < 200]
-        assert len(group) in (4, 8, 16) and group == q_loads, (name, q_loads)
-        dests = set()
-        for i in group:
-            dests |= regs_of(ins[i].split(",")[0])
-        assert len(dests) == 4 * len(group), name
-        # no instruction between the loads other than address arithmetic that stays off the destinations
-        for i in range(group[0], group[-1] + 1):
-            if i in group or ins[i].startswith(";;#ASM"):
-                continue
-            assert not (regs_of(ins[i]) & dests), (name, ins[i])
-        # after the last load: a manual wait must come before the first instruction that names a destination
-        seen_wait = False
-        for i in range(group[-1] + 1, len(ins)):
-            l = ins[i]
-            if l.startswith("s_waitcnt") and "vmcnt" in l:
-                seen_wait = True
-            if not l.startswith(";;#ASM") and regs_of(l) & dests:
-                assert seen_wait, (name, "destination of an in-flight Q load is used before any vmcnt wait", l)
-                break
-        else:
-            pytest.fail(f"{name}: the Q registers are never used")
+def asm_regions(ins):
+    """Yields the instruction lists of the inline-assembly statements of one kernel."""
+    cur = None
+    for l in ins:
+        if l.startswith(";;#ASMSTART"):
+            cur = []
+        elif l.startswith(";;#ASMEND"):
+            yield cur
+            cur = None
+        elif cur is not None:
+            cur.append(l)
 
 
-def test_no_scratch_or_stack_use_in_the_pipelined_loop(kernels):
-    """The 256-row kernels must keep their fused loop free of spill traffic: a scratch access there
-    is a vector-memory instruction the manual vmcnt accounting does not expect."""
-    for name, ins in kernels.items():
-        if "Li8ELi3ELb1" not in name:   # <.., 8 waves, K ring 3, pipelined, ..>
+def test_no_hand_issued_load_into_registers(kernels):
+    for name, (ins, _) in kernels.items():
+        for region in asm_regions(ins):
+            for l in region:
+                op = l.split()[0]
+                if op.startswith(("global_load", "buffer_load", "flat_load", "scratch_load")) and "_lds_" not in op:
+                    # the merge code's reads of other workgroups' partial results (device-scope, `sc1`) sit in one
+                    # statement with their own vmcnt(0), outputs bound by constraints: the compiler sees them complete
+                    assert "sc1" in l, (name, l)
+
+
+def test_the_whole_tile_pipelined_loop_has_no_spill_traffic(kernels):
+    """Scratch accesses are vector-memory instructions too: inside the fused loop of the 8-wave
+    kernels they would sit between the tile requests and the hand-counted waits and make every
+    wait longer than intended (never shorter: the counter retires in order)."""
+    checked = 0
+    for name, (ins, _) in kernels.items():
+        if "Li1ELi8ELi3ELi1ELb" not in name:   # <.., 32-row waves, 8 waves, K ring 3, pipelined, ..>
             continue
-        mfma_blocks, cur = [], []
+        blocks, cur = [], []
         for l in ins:
             if l.startswith("s_cbranch") or l.startswith("s_branch"):
-                mfma_blocks.append(cur)
+                blocks.append(cur)
                 cur = []
             else:
                 cur.append(l)
-        hot = [b for b in mfma_blocks if sum(1 for l in b if l.startswith("v_mfma")) >= 16 and any("v_exp_f32" in l for l in b)]
+        hot = [b for b in blocks if sum(1 for l in b if l.startswith("v_mfma")) >= 16 and any("v_exp_f32" in l for l in b)]
         assert hot, name
         for b in hot:
             assert not any(l.startswith("scratch_") or l.startswith("buffer_") for l in b), name
+        checked += 1
+    assert checked == 8
+
+
+def test_wide_kernels_hold_the_generated_loop_and_fit_the_register_file(kernels):
+    gen = _generator()
+    wide = {n: v for n, v in kernels.items() if "Li2ELi4ELi4ELi2ELb0" in n}   # <.., 64-row waves, 4 waves, K ring 4, wide, contiguous>
+    assert len(wide) == 4
+    for name, (ins, meta) in wide.items():
+        D = 128 if "Li128E" in name else 64
+        dtype = "bf16" if "IDF16b" in name else "f16"
+        want = [l.split(";")[0].strip() for l in gen.gen(D, dtype)]
+        want = [l for l in want if l and not l.endswith(":")]
+        regions = [r for r in asm_regions(ins) if len(r) > 1000]
+        assert len(regions) == 1, (name, [len(r) for r in asm_regions(ins)])
+        # `%=` in a label is the statement's number in the compiled code
+        got = [re.sub(r"(\.L\w+_)\d+$", r"\1%=", l) for l in regions[0] if not l.endswith(":")]
+        assert got == want, name   # the compiled loop IS the generator's text, register for register
+        # one wave per SIMD: accumulation and vector registers share a file of 512
+        assert meta["vgpr"] <= 512 and meta["agpr"] >= gen.A_Q + 8 * (D // 16), (name, meta)
+
+
+def test_committed_loop_text_is_what_the_generator_renders():
+    gen = _generator()
+    with open(os.path.join(fta_build.CSRC, "wide_loop_asm.inc")) as f:
+        assert f.read() == gen.render()
+
+
+def test_generator_rejects_undeclared_registers():
+    gen = _generator()
+    body, ops = gen.gen(128, "bf16"), gen.operands(128)
+    gen.verify(body, ops, "as rendered")
+    # a temporary the statement writes but does not list as clobbered
+    tmp = f'"s{gen.S_TMP + 7}"'
+    assert tmp in ops
+    with pytest.raises(AssertionError, match="writes undeclared"):
+        gen.verify(body, ops.replace(tmp + ", ", ""), "clobber dropped")
+    # a vector temporary
+    vt = f'"v{gen.V_T}"'
+    assert vt in ops
+    with pytest.raises(AssertionError, match="undeclared"):
+        gen.verify(body, ops.replace(vt + ", ", ""), "clobber dropped")
+    # an input the statement reads but the operand list does not bind
+    inp = f'"{{v{gen.V_KOFF}}}"(w_koff), '
+    assert inp in ops
+    with pytest.raises(AssertionError, match="reads undeclared"):
+        gen.verify(body, ops.replace(inp, ""), "input dropped")
+    # a write to an input-only operand
+    with pytest.raises(AssertionError, match="writes undeclared"):
+        gen.verify(body + [f"v_mov_b32 v{gen.V_KOFF}, 0"], ops, "input written")
+    # register tuples of vector registers start on an even register
+    with pytest.raises(AssertionError, match="misaligned"):
+        gen.verify(body + [f"v_mov_b64 v[{gen.V_T + 0 | 1}:{(gen.V_T + 0 | 1) + 1}], 0"], ops, "odd tuple")
+    # the masked-half statements go through the same check
+    for H in (0, 1):
+        gen.verify(gen.gen_masked(64, "f16", H), gen.operands_masked(64), "masked")
+        with pytest.raises(AssertionError, match="undeclared"):
+            gen.verify(gen.gen_masked(64, "f16", H), gen.operands_masked(64).replace(f'"v{gen.V_R}", ', ""), "masked, clobber dropped")

@@ -139,7 +139,7 @@ def test_reference_test_shape_fp16():
 SWEEP = [
     # bsz hq hkv  L   D   tmax dtype            lens
     (2, 4, 4, 1, 64, 100, torch.float16, [100, 33]),          # plain decode, one row
-    (2, 8, 2, 3, 128, 300, torch.bfloat16, [300, 1]),         # rows 12 < 16 -> shuffle
+    (2, 8, 2, 3, 128, 300, torch.bfloat16, [300, 1]),         # rows 12 < 16: MFMA kernel, rows past the unit's end blanked
     (1, 8, 2, 4, 128, 200, torch.bfloat16, [200]),            # rows 16 -> MFMA
     (3, 6, 3, 16, 64, 257, torch.float16, [0, 64, 257]),      # T=0, T multiple, T odd
     (2, 4, 1, 26, 128, 513, torch.float16, [513, 129]),       # rows 104, padded block
@@ -147,7 +147,7 @@ SWEEP = [
     (1, 2, 2, 128, 64, 90, torch.bfloat16, [90]),             # L 128: two tree tiles
     (1, 2, 1, 130, 128, 10, torch.float16, [10]),             # rows 260, ragged tree tiles
     (2, 4, 2, 8, 32, 150, torch.float16, [150, 20]),          # D 32 -> shuffle
-    (1, 4, 2, 8, 256, 150, torch.bfloat16, [131]),            # D 256 -> shuffle
+    (1, 4, 2, 8, 256, 150, torch.bfloat16, [131]),            # D 256: MFMA kernel, 128-row workgroups
     (2, 4, 2, 20, 256, 80, torch.float32, [80, 7]),           # fp32, D 256
     (1, 2, 2, 33, 32, 64, torch.float32, [64]),               # fp32, D 32, 3 row blocks of 16
 ]
