@@ -53,13 +53,24 @@ class FtaAppendArgs(C.Structure):
     ]
 
 
+LEN_BUCKETS = 16   # FTA_LEN_BUCKETS
+
+
 class FtaPlanOut(C.Structure):
     _fields_ = [
         ("kernel", C.c_int32), ("num_splits", C.c_int32), ("chunk", C.c_int32), ("rows_per_group", C.c_int32),
         ("rows_per_wg", C.c_int32), ("row_blocks", C.c_int32), ("num_workgroups", C.c_int32), ("counter_elems", C.c_int32),
         ("single_launch", C.c_int32), ("mfma_loop", C.c_int32),
         ("mid_o_elems", C.c_int64), ("mid_lse_elems", C.c_int64),
+        ("len_bound", C.c_int32 * LEN_BUCKETS), ("chunk_by_len", C.c_int32 * LEN_BUCKETS),
     ]
+
+    def chunk_for(self, max_len: int) -> int:
+        """Keys per split the kernels use for a batch whose longest sequence has max_len cached keys."""
+        for bound, chunk in zip(self.len_bound, self.chunk_by_len):
+            if max_len <= bound:
+                return chunk
+        return self.chunk_by_len[LEN_BUCKETS - 1]
 
 
 class FtaError(RuntimeError):

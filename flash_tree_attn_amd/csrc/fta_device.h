@@ -97,6 +97,45 @@ __device__ __forceinline__ WorkItem decode_work(const KernelParams& p, int id) {
   return w;
 }
 
+// Length of sequence b, clamped to the cache.
+__device__ __forceinline__ int clamped_len(const KernelParams& p, int b) {
+  const int64_t v = load_len(p.lens, p.len_is_i64, b);
+  return static_cast<int>(v < 0 ? 0 : (v > p.cache_len ? p.cache_len : v));
+}
+
+// Keys per split of this launch: the plan's entry for the batch's longest sequence
+// (len_bound ascends, so the lowest entry that covers max_len wins; lengths above the last
+// bound take the last entry).
+__device__ __forceinline__ int chunk_for(const KernelParams& p, int max_len) {
+  int c = p.chunk_by_len[FTA_LEN_BUCKETS - 1];
+#pragma unroll
+  for (int i = FTA_LEN_BUCKETS - 2; i >= 0; --i) c = max_len <= p.len_bound[i] ? p.chunk_by_len[i] : c;
+  return c;
+}
+
+// Maximum of `mine` over the block; every thread of the block must call it, once per kernel
+// (it keeps its per-wave slots until the block ends). Blocks of up to 1024 threads.
+__device__ __forceinline__ int block_max(int mine) {
+  __shared__ int s_wave_max[16];
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) mine = max(mine, __shfl_xor(mine, o, 64));
+  if ((threadIdx.x & 63) == 0) s_wave_max[threadIdx.x >> 6] = mine;
+  __syncthreads();
+  int m = 0;
+  for (int w = 0; w < static_cast<int>((blockDim.x + 63) >> 6); ++w) m = max(m, s_wave_max[w]);
+  return __builtin_amdgcn_readfirstlane(m);
+}
+
+// Keys per split of this launch, from the lengths of the whole batch; every thread of the
+// block must call it, once per kernel. Every workgroup of stage 1 and of stage 2 computes
+// the same value from the same lengths, so no workgroup has to tell another.
+__device__ __forceinline__ int batch_chunk(const KernelParams& p) {
+  if (p.bsz == 1) return chunk_for(p, clamped_len(p, 0));
+  int m = 0;
+  for (int i = threadIdx.x; i < p.bsz; i += blockDim.x) m = max(m, clamped_len(p, i));
+  return chunk_for(p, block_max(m));
+}
+
 // Longest-first dispatch for ragged batches. Workgroup ids are handed out in order, and
 // round-robin at every level of the machine (XCD, then shader engine), so any run of
 // consecutive ids should carry near-equal work and the heaviest items should come first.
@@ -104,29 +143,37 @@ __device__ __forceinline__ WorkItem decode_work(const KernelParams& p, int id) {
 // first every full chunk (all equal work; sequence-major), then the last chunk of every
 // sequence (partial chunk + tree block) in descending size; what remains of the grid has
 // nothing to do. No host look at the lengths and no atomics: every workgroup recomputes
-// the order from the bsz lengths in one LDS pass (and gets its sequence's clamped length
-// back with it). Batches of one sequence or beyond
+// the order from the bsz lengths in LDS (and gets its sequence's clamped length and the
+// launch's chunk length back with it). Batches of one sequence or beyond
 // kMaxOrderedBatch keep the identity order. Returns false if the item is empty. Must be
 // called by all threads of the block.
 constexpr int kMaxOrderedBatch = 256;
-__device__ __forceinline__ bool item_by_order(const KernelParams& p, int k, int* batch, int* split, int* len) {
+__device__ __forceinline__ bool item_by_order(const KernelParams& p, int k, int* batch, int* split, int* len, int* chunk_out) {
   if (p.bsz == 1 || p.bsz > kMaxOrderedBatch) {
+    const int chunk = batch_chunk(p);
+    *chunk_out = chunk;
     *batch = k / p.num_splits;
     *split = k % p.num_splits;
-    const int64_t v = load_len(p.lens, p.len_is_i64, *batch);
-    *len = static_cast<int>(v < 0 ? 0 : (v > p.cache_len ? p.cache_len : v));
+    *len = clamped_len(p, *batch);
     return true;
   }
   __shared__ int s_nsp[kMaxOrderedBatch];
   __shared__ int s_tail[kMaxOrderedBatch];
   __shared__ int s_pick[3];
   const int t = threadIdx.x;
+  int longest = 0;
   for (int i = t; i < p.bsz; i += blockDim.x) {
-    const int64_t v = load_len(p.lens, p.len_is_i64, i);
-    const int len = static_cast<int>(v < 0 ? 0 : (v > p.cache_len ? p.cache_len : v));
-    const int n = splits_for(len, p.chunk, p.num_splits);
+    const int len = clamped_len(p, i);
+    s_tail[i] = len;   // parked here until the chunk is known; the same thread comes back for it
+    longest = max(longest, len);
+  }
+  const int chunk = chunk_for(p, block_max(longest));
+  *chunk_out = chunk;
+  for (int i = t; i < p.bsz; i += blockDim.x) {
+    const int len = s_tail[i];
+    const int n = splits_for(len, chunk, p.num_splits);
     s_nsp[i] = n;
-    s_tail[i] = len - (n - 1) * p.chunk;
+    s_tail[i] = len - (n - 1) * chunk;
   }
   if (t == 0) s_pick[0] = -1;
   __syncthreads();
@@ -143,7 +190,7 @@ __device__ __forceinline__ bool item_by_order(const KernelParams& p, int k, int*
     if (full || k - total == rank) {
       s_pick[0] = i;
       s_pick[1] = full ? k - before : s_nsp[i] - 1;
-      s_pick[2] = mine + (s_nsp[i] - 1) * p.chunk;   // the (clamped) length, so that callers need not load it again
+      s_pick[2] = mine + (s_nsp[i] - 1) * chunk;   // the (clamped) length, so that callers need not load it again
     }
   }
   __syncthreads();

@@ -5,6 +5,7 @@
 
 #include <cmath>
 #include <algorithm>
+#include <cstdint>
 #include <cstdlib>
 
 #include "fta_internal.h"
@@ -133,57 +134,82 @@ int plan(const fta_args& a, int num_cus, fta_plan_out* out) {
   // fp32 partials written and read back. Few long chunks win over many short ones:
   // the fixed part is worth 7-10 tiles.
   const int64_t target = static_cast<int64_t>(num_cus) * wg_per_cu;
-  const int64_t min_chunk = std::max<int64_t>(gran, 4 * kKeyTile);
-  const int64_t s_max = std::max<int64_t>(1, std::min<int64_t>(64, std::max<int64_t>(t_cap, 1) / min_chunk));
-  const double fixed_us = kernel != FTA_KERNEL_MFMA ? 5.0 : wg_per_cu > 1 ? 12.0 : 20.0;   // partly hidden behind co-resident workgroups
-  // per workgroup and 64-key tile, with the CU fully occupied: the pipelined 256-row
-  // variant alone on its CU; the plain 128-row variant next to a second workgroup, by
-  // the number of its waves that hold rows; the shuffle kernel with four workgroups per CU.
-  const int live_waves = std::min(4, static_cast<int>(cdiv(std::min(rows, rows_per_wg), 32)));
-  const double tile_us = kernel != FTA_KERNEL_MFMA ? 5.0 : rows_per_wg > 128 ? 2.85 : (1.0 + 0.7 * live_waves) * (a.head_dim > 128 ? 2.0 : 1.0);
-  const double tree_tiles = 3.0 * cdiv(a.q_len, kKeyTile);
-  const double tail_share = a.bsz > 1 ? 0.25 : 0.0;
-  const double partial_mb = 4e-6 * a.bsz * a.num_q_heads * a.q_len * a.head_dim;  // MB per split slot
-  int64_t splits = 1;
-  double best = 0.0;
-  double cost_of[65];
-  for (int64_t cand = 1; cand <= s_max; ++cand) {
-    const double tiles = std::ceil((std::max<int64_t>(t_cap, 1) / static_cast<double>(kKeyTile) + tree_tiles) / cand);
-    const double wg_us = fixed_us + tile_us * tiles;
-    const double rounds = static_cast<double>(cdiv(work_items * cand, target));
-    const double merge_us = cand > 1 ? 6.0 + cand * partial_mb / 2.0 : 0.0;   // written once, read once, at ~4-5 TB/s
-    const double cost = (rounds + tail_share) * wg_us + merge_us;
-    cost_of[cand] = cost;
-    if (cand == 1 || cost < best * 0.98) {  // a larger count has to win by 2 %
-      best = cost;
-      splits = cand;
+  struct Cut { int64_t splits, chunk; };
+  // The cut for sequences of up to t_len cached keys, with at most s_limit splits (a forced
+  // count is only held to the limit when `limit_forced`).
+  auto cut_for = [&](int64_t t_len, int64_t s_limit, bool limit_forced) -> Cut {
+    t_len = std::max<int64_t>(t_len, 1);
+    const int64_t forced_limit = limit_forced ? s_limit : INT64_MAX;
+    const int64_t min_chunk = std::max<int64_t>(gran, 4 * kKeyTile);
+    const int64_t s_max = std::max<int64_t>(1, std::min<int64_t>(s_limit, t_len / min_chunk));
+    const double fixed_us = kernel != FTA_KERNEL_MFMA ? 5.0 : wg_per_cu > 1 ? 12.0 : 20.0;   // partly hidden behind co-resident workgroups
+    // per workgroup and 64-key tile, with the CU fully occupied: the pipelined 256-row
+    // variant alone on its CU; the plain 128-row variant next to a second workgroup, by
+    // the number of its waves that hold rows; the shuffle kernel with four workgroups per CU.
+    const int live_waves = std::min(4, static_cast<int>(cdiv(std::min(rows, rows_per_wg), 32)));
+    const double tile_us = kernel != FTA_KERNEL_MFMA ? 5.0 : rows_per_wg > 128 ? 2.85 : (1.0 + 0.7 * live_waves) * (a.head_dim > 128 ? 2.0 : 1.0);
+    const double tree_tiles = 3.0 * cdiv(a.q_len, kKeyTile);
+    const double tail_share = a.bsz > 1 ? 0.25 : 0.0;
+    const double partial_mb = 4e-6 * a.bsz * a.num_q_heads * a.q_len * a.head_dim;  // MB per split slot
+    int64_t splits = 1;
+    double best = 0.0;
+    double cost_of[65];
+    for (int64_t cand = 1; cand <= s_max; ++cand) {
+      const double tiles = std::ceil((t_len / static_cast<double>(kKeyTile) + tree_tiles) / cand);
+      const double wg_us = fixed_us + tile_us * tiles;
+      const double rounds = static_cast<double>(cdiv(work_items * cand, target));
+      const double merge_us = cand > 1 ? 6.0 + cand * partial_mb / 2.0 : 0.0;   // written once, read once, at ~4-5 TB/s
+      const double cost = (rounds + tail_share) * wg_us + merge_us;
+      cost_of[cand] = cost;
+      if (cand == 1 || cost < best * 0.98) {  // a larger count has to win by 2 %
+        best = cost;
+        splits = cand;
+      }
     }
+    // A batch whose workgroups all fit the machine at once is only balanced if its sequences
+    // are equally long, and the lengths are not known here: the longest sequence then sets the
+    // time while most CUs idle. For batches of 8 and more, up to twice the splits are taken
+    // where the model prices that at no more than 10 % on an equal-length batch. Measured over
+    // split sweeps of 76 ragged and 112 equal-length shapes: -6 % on the ragged ones on
+    // average (worst case 2.1x -> 1.3x of the best split count), +1 % on the equal-length ones.
+    if (a.bsz >= 8 && a.head_dim <= 128 && work_items * splits <= target) {   // head_dim 256: the model is not calibrated well enough
+      const int64_t chosen = splits;
+      for (int64_t cand = chosen + 1; cand <= std::min<int64_t>(2 * chosen, s_max); ++cand)
+        if (cost_of[cand] <= cost_of[chosen] * 1.10) splits = cand;
+    }
+    if (a.force_splits > 0) splits = std::min<int64_t>(a.force_splits, forced_limit);
+    if (env_knobs().force_splits > 0) splits = std::min<int64_t>(env_knobs().force_splits, forced_limit);
+    // Never more splits than blocks of the reference granularity, so that a scratch
+    // buffer sized like the reference's (flash_tree_attn.py:274-281) always fits.
+    splits = std::min<int64_t>(splits, std::max<int64_t>(1, cdiv(t_len, gran)));
+    // The split that owns the end of a sequence also processes the tree block (a masked,
+    // latency-bound step worth about three cache tiles per tree tile): count it as extra
+    // keys when cutting chunks, so that the last split of a full-length sequence gets a
+    // correspondingly shorter cache range.
+    const int64_t tree_weight = env_knobs().tree_tile_weight >= 0 ? env_knobs().tree_tile_weight : 3;
+    const int64_t tree_keys = splits > 1 ? tree_weight * kKeyTile * cdiv(a.q_len, kKeyTile) : 0;
+    int64_t chunk = cdiv(cdiv(t_len + tree_keys, splits), gran) * gran;
+    if ((splits - 1) * chunk >= t_len) chunk = cdiv(cdiv(t_len, splits), gran) * gran;
+    splits = std::max<int64_t>(1, cdiv(t_len, chunk));
+    return Cut{splits, chunk};
+  };
+  // The grid and the scratch buffers are sized for the length cap. The lengths themselves are
+  // only known on the device, and a cap far above them (a cache allocated for the longest
+  // context the server admits, a page table's full width) would leave most splits without
+  // keys. The kernels therefore take the chunk from a table by the batch's longest sequence:
+  // the cut this model makes for that length within the cap's split count. Bounds fall
+  // from the cap in steps of 3/4 and 2/3 (1, 3/4, 1/2, 3/8, ...), so the table entry is for
+  // a length at most a third above the real one; a batch at the cap gets the cap's own cut.
+  const int64_t cap = std::max<int64_t>(t_cap, 1);
+  const Cut cap_cut = cut_for(cap, 64, false);
+  const int64_t splits = cap_cut.splits, chunk = cap_cut.chunk;
+  for (int i = 0; i < FTA_LEN_BUCKETS; ++i) {
+    const int k = FTA_LEN_BUCKETS - 1 - i;   // steps below the cap
+    const int64_t fraction = cdiv((k % 2 ? 3 : 1) * cap, int64_t{1} << (k % 2 ? (k + 3) / 2 : k / 2));
+    const int64_t bound = k == 0 ? cap : std::min(cap, cdiv(fraction, gran) * gran);
+    out->len_bound[i] = static_cast<int32_t>(bound);
+    out->chunk_by_len[i] = static_cast<int32_t>(k == 0 ? chunk : cut_for(bound, splits, true).chunk);
   }
-  // A batch whose workgroups all fit the machine at once is only balanced if its sequences
-  // are equally long, and the lengths are not known here: the longest sequence then sets the
-  // time while most CUs idle. For batches of 8 and more, up to twice the splits are taken
-  // where the model prices that at no more than 10 % on an equal-length batch. Measured over
-  // split sweeps of 76 ragged and 112 equal-length shapes: -6 % on the ragged ones on
-  // average (worst case 2.1x -> 1.3x of the best split count), +1 % on the equal-length ones.
-  if (a.bsz >= 8 && a.head_dim <= 128 && work_items * splits <= target) {   // head_dim 256: the model is not calibrated well enough
-    const int64_t chosen = splits;
-    for (int64_t cand = chosen + 1; cand <= std::min<int64_t>(2 * chosen, s_max); ++cand)
-      if (cost_of[cand] <= cost_of[chosen] * 1.10) splits = cand;
-  }
-  if (a.force_splits > 0) splits = a.force_splits;
-  if (env_knobs().force_splits > 0) splits = env_knobs().force_splits;
-  // Never more splits than blocks of the reference granularity, so that a scratch
-  // buffer sized like the reference's (flash_tree_attn.py:274-281) always fits.
-  splits = std::min<int64_t>(splits, std::max<int64_t>(1, cdiv(t_cap, gran)));
-  // The split that owns the end of a sequence also processes the tree block (a masked,
-  // latency-bound step worth about three cache tiles per tree tile): count it as extra
-  // keys when cutting chunks, so that the last split of a full-length sequence gets a
-  // correspondingly shorter cache range.
-  const int64_t tree_weight = env_knobs().tree_tile_weight >= 0 ? env_knobs().tree_tile_weight : 3;
-  const int64_t tree_keys = splits > 1 ? tree_weight * kKeyTile * cdiv(a.q_len, kKeyTile) : 0;
-  int64_t chunk = cdiv(cdiv(std::max<int64_t>(t_cap, 1) + tree_keys, splits), gran) * gran;
-  if ((splits - 1) * chunk >= std::max<int64_t>(t_cap, 1)) chunk = cdiv(cdiv(std::max<int64_t>(t_cap, 1), splits), gran) * gran;
-  splits = std::max<int64_t>(1, cdiv(std::max<int64_t>(t_cap, 1), chunk));
 
   out->kernel = kernel;
   out->num_splits = static_cast<int32_t>(splits);
@@ -291,6 +317,10 @@ int decode_impl(const fta_args* args, void* hip_stream, int stages) {
   p.wide_loop = pl.mfma_loop;
   p.bsz = a.bsz; p.num_q_heads = a.num_q_heads; p.q_len = a.q_len; p.cache_len = a.cache_len;
   p.chunk = pl.chunk; p.num_splits = pl.num_splits;
+  for (int i = 0; i < FTA_LEN_BUCKETS; ++i) {
+    p.len_bound[i] = pl.len_bound[i];
+    p.chunk_by_len[i] = pl.chunk_by_len[i];
+  }
   p.heads_per_unit = pl.rows_per_group / a.q_len;
   p.units = a.num_q_heads / p.heads_per_unit;
   p.kv_group = a.num_q_heads / a.num_kv_heads;

@@ -31,7 +31,7 @@ struct KernelParams {
   int32_t num_q_heads;
   int32_t q_len;
   int32_t cache_len;
-  int32_t chunk;
+  int32_t chunk;          // keys per split at the length cap (the last entry of chunk_by_len)
   int32_t num_splits;
   int32_t heads_per_unit;
   int32_t units;          // num_q_heads / heads_per_unit
@@ -46,6 +46,8 @@ struct KernelParams {
   int32_t page_shift;     // log2(page size) when block_table is set
   int32_t wide_loop;      // 256-row workgroups: 4 waves x 64 rows with the half-tile loop instead of 8 waves x 32 rows
   float scale_log2;       // sm_scale * log2(e)
+  int32_t len_bound[FTA_LEN_BUCKETS];     // ascending; the chunk of a launch is chunk_by_len[first i with max length <= len_bound[i]]
+  int32_t chunk_by_len[FTA_LEN_BUCKETS];
 
   int64_t q_stride[3];
   int64_t k_stride[3];

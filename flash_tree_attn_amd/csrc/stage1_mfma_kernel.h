@@ -231,12 +231,12 @@ stage1_mfma_kernel(const KernelParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   const WorkItem w = decode_work(p, blockIdx.x);
-  int b, split, T_b;
-  if (!item_by_order(p, w.item, &b, &split, &T_b)) return;
-  const int S_b = splits_for(T_b, p.chunk, p.num_splits);
+  int b, split, T_b, chunk;   // chunk: keys per split of this launch, from the batch's longest sequence
+  if (!item_by_order(p, w.item, &b, &split, &T_b, &chunk)) return;
+  const int S_b = splits_for(T_b, chunk, p.num_splits);
   if (split >= S_b) return;
-  const int kv_start = split * p.chunk;
-  const int kv_end = (split == p.num_splits - 1) ? T_b : min(T_b, kv_start + p.chunk);
+  const int kv_start = split * chunk;
+  const int kv_end = (split == p.num_splits - 1) ? T_b : min(T_b, kv_start + chunk);
   const bool owns_tree = (split == S_b - 1);
 
   const int tid = threadIdx.x;

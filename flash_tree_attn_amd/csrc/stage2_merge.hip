@@ -33,6 +33,7 @@ template <typename T, int D>
 __global__ void __launch_bounds__(256) stage2_merge_kernel(const KernelParams p) {
   constexpr int kThreadsPerRow = D / 4;
   constexpr int kRowsPerBlock = 256 / kThreadsPerRow;
+  const int chunk = batch_chunk(p);   // the same cut stage 1 made (block-wide: before any thread leaves)
   const int64_t total_rows = static_cast<int64_t>(p.bsz) * p.num_q_heads * p.q_len;
   const int64_t row = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + threadIdx.x / kThreadsPerRow;
   if (row >= total_rows) return;
@@ -41,9 +42,7 @@ __global__ void __launch_bounds__(256) stage2_merge_kernel(const KernelParams p)
   const int head = static_cast<int>((row / p.q_len) % p.num_q_heads);
   const int b = static_cast<int>(row / (static_cast<int64_t>(p.q_len) * p.num_q_heads));
 
-  int64_t t64 = load_len(p.lens, p.len_is_i64, b);
-  const int T_b = static_cast<int>(t64 < 0 ? 0 : (t64 > p.cache_len ? p.cache_len : t64));
-  const int S_b = splits_for(T_b, p.chunk, p.num_splits);
+  const int S_b = splits_for(clamped_len(p, b), chunk, p.num_splits);
 
   const float* lse = p.mid_lse + b * p.mid_lse_stride[0] + head * p.mid_lse_stride[1] + i;
   const float* mo = p.mid_o + b * p.mid_o_stride[0] + head * p.mid_o_stride[1] + i * p.mid_o_stride[3] + d;

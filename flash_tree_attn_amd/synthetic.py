@@ -46,6 +46,8 @@ CONFIGS: Dict[str, Config] = {
     "decode1_gqa4_bf16": Config("decode1_gqa4_bf16", 64, 32, 8, 128, 1, 4096, torch.bfloat16, "full", "chain"),
     # the shape of the reference's own test (flash_tree_attn.py:416,435: Z 32, H 32, N_CTX 4096, D 128, q_len 128, block 128)
     "reftest_mha_fp16": Config("reftest_mha_fp16", 32, 32, 32, 128, 128, 4096, torch.float16, "full", "random", 128),
+    # the headline shape inside a cache allocated for 64K positions: the lengths, not the capacity, must set the cut
+    "cfg3_in_64k_cache_bf16": Config("cfg3_in_64k_cache_bf16", 8, 32, 8, 128, 64, 65536, torch.bfloat16, "uniform:8192:8192", "random"),
     # head_dim 256 (two query heads per cache head), tree of 64
     "d256_gqa2_bf16": Config("d256_gqa2_bf16", 8, 16, 8, 256, 64, 8192, torch.bfloat16, "full", "random"),
 }

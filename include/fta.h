@@ -111,7 +111,8 @@ typedef struct fta_args {
   int32_t cache_len;        /* k_cache.size(2) */
   int32_t v_cache_len;      /* v_cache.size(2), must equal cache_len */
   int32_t block_size;       /* the reference's split granularity (flash_tree_attn.py:268) */
-  int32_t max_seq_len_hint; /* max_seq_len_in_batch, or 0 when the caller gave none */
+  int32_t max_seq_len_hint; /* max_seq_len_in_batch: an upper bound of kv_seq_len that sizes the grid and the scratch, or
+                               0 = cache_len. How the keys are cut into chunks follows the real lengths (fta_plan_out) */
   int32_t mid_splits;       /* size(2) of mid_o / mid_lse, 0 when they are NULL */
   int32_t dtype;            /* fta_dtype of q/k/v/cur/out */
   int32_t len_dtype;        /* fta_len_dtype of kv_seq_len */
@@ -134,11 +135,13 @@ typedef struct fta_args {
   int64_t block_table_stride; /* batch stride of block_table */
 } fta_args;
 
+#define FTA_LEN_BUCKETS 16
+
 /* What the split heuristic decided for one fta_args (pure host arithmetic). */
 typedef struct fta_plan_out {
   int32_t kernel;         /* fta_kernel */
   int32_t num_splits;     /* grid extent along the KV sequence; 1 = single pass, no scratch, no stage 2 */
-  int32_t chunk;          /* keys per split; a multiple of block_size and of the kernel's key tile */
+  int32_t chunk;          /* keys per split for a batch at the length cap; a multiple of block_size and of the kernel's key tile */
   int32_t rows_per_group; /* kv_group_num * q_len: query rows that share one K/V stream */
   int32_t rows_per_wg;    /* query rows one workgroup holds */
   int32_t row_blocks;     /* ceil(rows_per_group / rows_per_wg) */
@@ -150,6 +153,14 @@ typedef struct fta_plan_out {
   int32_t mfma_loop;      /* MFMA kernel, 256-row workgroups: 0 = 8 waves x 32 rows, 1 = 4 waves x 64 rows (half-tile loop) */
   int64_t mid_o_elems;    /* float32 elements a dense mid_o for this plan needs */
   int64_t mid_lse_elems;
+  /* Keys per split by the batch's longest sequence: the kernels read the lengths, find the first i
+   * with max(kv_seq_len) <= len_bound[i] (the last entry if none) and cut every sequence into chunks
+   * of chunk_by_len[i] keys, so that a length cap far above the real lengths (a cache allocated for
+   * the longest admissible context, a page table's full width) does not leave most splits empty.
+   * len_bound ascends to the cap; chunk_by_len[FTA_LEN_BUCKETS - 1] == chunk. Sequence b then fills
+   * min(num_splits, max(1, ceil(kv_seq_len[b] / that chunk))) split slots of mid_o / mid_lse. */
+  int32_t len_bound[FTA_LEN_BUCKETS];
+  int32_t chunk_by_len[FTA_LEN_BUCKETS];
 } fta_plan_out;
 
 /* ABI version of the loaded library (== FTA_ABI_VERSION it was built with). */

@@ -54,7 +54,7 @@ def test_header_symbols_exported(fta_lib):
 def test_struct_layout_matches_header(fta_lib, tmp_path):
     # 12 pointers, 18 int32 + 1 float (padded to 8), 9 stride arrays (8 of 3 + 1 of 4 int64), 1 int64
     assert C.sizeof(_lib.FtaArgs) == 12 * 8 + 20 * 4 + (8 * 3 + 4) * 8 + 8
-    assert C.sizeof(_lib.FtaPlanOut) == 10 * 4 + 2 * 8
+    assert C.sizeof(_lib.FtaPlanOut) == 10 * 4 + 2 * 8 + 2 * _lib.LEN_BUCKETS * 4
     # ... and field by field against what a C compiler makes of include/fta.h
     fields = [n for n, _ in _lib.FtaArgs._fields_]
     plan_fields = [n for n, _ in _lib.FtaPlanOut._fields_]
@@ -214,6 +214,60 @@ def test_plan_overrides(fta_lib):
     assert st == 0 and pl.kernel == _lib.KERNEL_SHUFFLE and pl.rows_per_wg == 16
     st, _ = plan(fta_lib, base_args(force_kernel=_lib.KERNEL_MFMA, dtype=_lib.FTA_F32))
     assert st == -9
+
+
+def _live_workgroups(pl, lengths, units_x_row_blocks):
+    """Stage-1 workgroups that have keys to process, the way the kernels count them."""
+    chunk = pl.chunk_for(max(lengths))
+    return sum(min(pl.num_splits, max(1, -(-t // chunk))) for t in lengths) * units_x_row_blocks
+
+
+@pytest.mark.parametrize("kw", [
+    dict(), dict(bsz=1), dict(bsz=3, q_len=16), dict(head_dim=64, dtype=_lib.FTA_F16), dict(q_len=1, num_q_heads=8, num_kv_heads=8, cur_heads=8),
+    dict(dtype=_lib.FTA_F32), dict(block_size=128), dict(force_splits=7), dict(cache_len=100, v_cache_len=100), dict(cache_len=0, v_cache_len=0),
+    dict(max_seq_len_hint=3000), dict(head_dim=256, q_len=8),
+])
+@pytest.mark.parametrize("capacity", [None, 131072])
+def test_chunk_table_invariants(fta_lib, kw, capacity):
+    kw = dict(kw)
+    if capacity and "cache_len" not in kw:
+        kw.update(cache_len=capacity, v_cache_len=capacity)
+    a = base_args(**kw)
+    st, pl = plan(fta_lib, a)
+    assert st == 0
+    cap = max(1, min(a.cache_len, a.max_seq_len_hint) if a.max_seq_len_hint else a.cache_len)
+    bounds, chunks = list(pl.len_bound), list(pl.chunk_by_len)
+    gran = max(a.block_size, 64)
+    assert bounds == sorted(bounds) and bounds[-1] == cap and chunks[-1] == pl.chunk
+    for i, (bound, chunk) in enumerate(zip(bounds, chunks)):
+        assert 1 <= bound <= cap
+        assert chunk > 0 and chunk % gran == 0                      # whole key tiles and whole reference blocks
+        assert pl.num_splits * chunk >= bound                       # the grid's split slots cover every length of the bucket
+        assert -(-bound // chunk) <= pl.num_splits
+        if i:
+            assert bound * 2 <= bounds[i - 1] * 3 + 3 * gran        # steps of at most 3/2 (plus rounding to whole blocks)
+        assert pl.chunk_for(bound) == chunks[bounds.index(bound)]   # equal bounds: the first entry serves
+    assert pl.chunk_for(cap + 1) == pl.chunk and pl.chunk_for(0) == chunks[0]
+
+
+def test_chunks_follow_the_lengths_not_the_capacity(fta_lib):
+    """A cache far larger than the sequences in it (or a wide page table) must not leave the
+    grid idle: for the headline shape with 8192 live keys the cut is the one a cache of
+    exactly 8192 gets, whatever the capacity, and one sequence still spreads over the machine."""
+    st, exact = plan(fta_lib, base_args())
+    assert st == 0 and (exact.num_splits, exact.chunk) == (4, 2112)
+    for capacity in (8192, 12288, 16384, 65536, 131072):
+        st, pl = plan(fta_lib, base_args(cache_len=capacity, v_cache_len=capacity))
+        assert st == 0
+        live = _live_workgroups(pl, [8192] * 8, 8)
+        assert 192 <= live <= 256, (capacity, pl.num_splits, pl.chunk_for(8192), live)
+        assert pl.chunk_for(8192) <= 2 * 2112
+    st, one = plan(fta_lib, base_args(bsz=1, cache_len=131072, v_cache_len=131072))
+    st2, one_exact = plan(fta_lib, base_args(bsz=1))
+    assert st == 0 and st2 == 0
+    assert _live_workgroups(one, [8192], 8) >= 0.6 * _live_workgroups(one_exact, [8192], 8)
+    # and a short batch in the big cache is not shredded either: chunks stay at four key tiles or more
+    assert one.chunk_for(700) >= 256
 
 
 def test_plan_of_the_64_row_wave_loop(fta_lib):

@@ -1,0 +1,340 @@
+"""GPU tests of what the library exports beyond the one-call path, and of how much margin the
+one-call path has:
+
+* `fta_decode_stage1` alone: every live slot of the scratch buffers against the oracle's
+  partial for that split (flash_tree_attn.py:49-144; the split that owns the end of a
+  sequence also holds the tree block, flash_tree_attn.py:367-373);
+* `fta_decode_stage2` alone on oracle-made partials against `stage2_merge_oracle`
+  (flash_tree_attn.py:174-211), with sequences that fill fewer slots than the grid has;
+* caches much larger than the sequences in them (the cut must follow the lengths);
+* the 64-row-wave MFMA loop, which only runs when asked for;
+* head_dim 256 through the merge inside stage 1 and on paged caches;
+* one sequence x two heads of the headline workload against the fp64 oracle on the CPU;
+* the largest error of each benchmark configuration as a share of the tolerance.
+
+The helper that predicts the partials is itself checked on the CPU: its partials, merged,
+must be the whole-path oracle."""
+import math
+
+import pytest
+import torch
+
+from flash_tree_attn_amd import _lib
+from flash_tree_attn_amd.synthetic import CONFIGS, make_inputs
+from flash_tree_attn_amd.tree_mask import additive_mask_from_parents, random_tree_parents
+from oracle.tree_attn_oracle import (_expand_heads, _mask_for, stage1_partial_oracle, stage2_merge_oracle, tree_attention_oracle,
+                                     tree_block_oracle)
+
+TOL = {torch.float16: dict(atol=2e-3, rtol=1e-2), torch.bfloat16: dict(atol=2e-3, rtol=1e-2),
+       torch.float32: dict(atol=2e-5, rtol=1e-4)}
+DEV = "cuda"
+
+
+def make(seed, bsz, hq, hkv, L, D, tmax, dtype, lens, device=DEV):
+    g = torch.Generator().manual_seed(seed)
+    r = lambda *s: torch.randn(*s, generator=g).to(dtype).to(device)
+    x = dict(q=r(bsz, hq, L, D), k_cache=r(bsz, hkv, tmax, D), v_cache=r(bsz, hkv, tmax, D),
+             current_k=r(bsz, hkv, L, D), current_v=r(bsz, hkv, L, D))
+    x["mask"] = additive_mask_from_parents(random_tree_parents(L, g), device=device)
+    x["kv_seq_len"] = torch.as_tensor(lens, dtype=torch.int64).to(device)
+    x["kv_group_num"] = hq // hkv
+    return x
+
+
+def oracle(x, dtype=torch.float32):
+    return tree_attention_oracle(x["q"], x["k_cache"], x["v_cache"], x["current_k"], x["current_v"], x["mask"],
+                                 x["kv_seq_len"], None, x["kv_group_num"], dtype=dtype)
+
+
+def prepare(x, **kw):
+    from flash_tree_attn_amd import flash_decoding as fd
+    return fd.prepare(x["q"], x["k_cache"], x["v_cache"], x["current_k"], x["current_v"], x["mask"], x["kv_seq_len"], 64,
+                      kv_group_num=x["kv_group_num"], **kw)
+
+
+def check(out, ref, dtype):
+    assert out.dtype == dtype
+    assert torch.isfinite(out).all()
+    torch.testing.assert_close(out.float(), ref.float(), **TOL[dtype])
+
+
+def live_splits(t_b, chunk, num_splits):
+    """Split slots sequence b fills: ceil(T_b / chunk), at least one (the tree block needs a home), at most the grid's."""
+    return min(num_splits, max(1, -(-t_b // chunk)))
+
+
+def expected_partials(x, b, chunk, num_splits, dtype=torch.float32):
+    """[(o [Hq, L, D], lse [Hq, L])] for the live splits of sequence b: split s covers cache keys
+    [s * chunk, (s + 1) * chunk) (the grid's last split runs to the end), and the last live split also
+    attends to the tree keys under the mask. Partials are normalised, lse is the natural-log sum."""
+    bsz, hq, L, D = x["q"].shape
+    scale = 1.0 / math.sqrt(D)
+    t_b = min(max(int(x["kv_seq_len"][b]), 0), x["k_cache"].size(2))
+    qb = x["q"][b].to(dtype)
+    kb = _expand_heads(x["k_cache"][b, :, :t_b].to(dtype), hq)
+    vb = _expand_heads(x["v_cache"][b, :, :t_b].to(dtype), hq)
+    s_b = live_splits(t_b, chunk, num_splits)
+    parts = []
+    for s in range(s_b):
+        lo = s * chunk
+        hi = t_b if s == num_splits - 1 else min(t_b, lo + chunk)
+        pieces = []
+        if hi > lo:
+            pieces.append(stage1_partial_oracle(qb, kb, vb, lo, hi, scale))
+        if s == s_b - 1:
+            pieces.append(tree_block_oracle(qb, _expand_heads(x["current_k"][b].to(dtype), hq), _expand_heads(x["current_v"][b].to(dtype), hq),
+                                            _mask_for(x["mask"], b, bsz, hq, L, dtype), scale))
+        parts.append(stage2_merge_oracle([p[0] for p in pieces], [p[1] for p in pieces]))
+    return parts
+
+
+@pytest.mark.parametrize("lens,chunk,num_splits", [([300, 64, 0], 128, 4), ([500, 499], 64, 3), ([1], 64, 1), ([130], 64, 8)])
+def test_predicted_partials_merge_to_the_whole_path_oracle(lens, chunk, num_splits):
+    x = make(5, len(lens), 4, 2, 6, 32, 512, torch.float32, lens, device="cpu")
+    ref = oracle(x, torch.float64)
+    for b, t_b in enumerate(lens):
+        parts = expected_partials(x, b, chunk, num_splits, torch.float64)
+        assert len(parts) == live_splits(t_b, chunk, num_splits)
+        merged, _ = stage2_merge_oracle([p[0] for p in parts], [p[1] for p in parts])
+        torch.testing.assert_close(merged, ref[b], atol=1e-12, rtol=1e-10)
+
+
+# ---------------------------------------------------------------- stage 1 alone
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [
+    # bsz hq hkv  L   D   tmax  dtype           lens               splits
+    (2, 8, 2, 64, 128, 1500, torch.bfloat16, [1500, 400], 4),          # 256-row MFMA workgroups; the short sequence fills one slot
+    (3, 8, 2, 16, 64, 900, torch.float16, [900, 0, 333], 3),           # 128-row MFMA workgroups, an empty cache
+    (2, 4, 2, 8, 256, 700, torch.bfloat16, [700, 350], 2),             # head_dim 256
+    (2, 4, 4, 3, 32, 600, torch.float32, [600, 130], 4),               # shuffle kernel, fp32
+    (2, 8, 2, 64, 128, 8192, torch.bfloat16, [700, 300], 4),           # a cache far larger than the sequences: chunks follow the lengths
+])
+def test_stage1_alone_fills_the_slots_the_oracle_predicts(shape):
+    bsz, hq, hkv, L, D, tmax, dtype, lens, splits = shape
+    x = make(71, bsz, hq, hkv, L, D, tmax, dtype, lens)
+    pc = prepare(x, _force_splits=splits)
+    S = pc.plan.num_splits
+    assert S > 1 and pc.mid_output.shape == (bsz, hq, S, L, D) and pc.mid_output_lse.shape == (bsz, hq, S, L)
+    nan = float("nan")
+    pc.mid_output.fill_(nan), pc.mid_output_lse.fill_(nan), pc.output.fill_(nan)
+    pc.run_stage1()
+    torch.cuda.synchronize()
+    assert torch.isnan(pc.output).all()                     # the first half alone leaves `out` alone
+    chunk = pc.plan.chunk_for(max(min(t, tmax) for t in lens))
+    if max(lens) * 4 < tmax:
+        assert chunk < pc.plan.chunk                        # the cut is the lengths', not the capacity's
+    for b, t_b in enumerate(lens):
+        parts = expected_partials(x, b, chunk, S)
+        assert len(parts) == live_splits(t_b, chunk, S)
+        for s, (o_ref, lse_ref) in enumerate(parts):
+            got_o, got_lse = pc.mid_output[b, :, s], pc.mid_output_lse[b, :, s]
+            assert torch.isfinite(got_o).all(), (b, s)
+            torch.testing.assert_close(got_lse, lse_ref.float(), atol=2e-3, rtol=1e-4)
+            torch.testing.assert_close(got_o, o_ref.float(), **TOL[dtype])
+        for s in range(len(parts), S):                      # slots past the sequence's splits are never written
+            assert torch.isnan(pc.mid_output[b, :, s]).all() and torch.isnan(pc.mid_output_lse[b, :, s]).all(), (b, s)
+    # ... and the second half finishes the call from exactly these buffers
+    pc.run_stage2()
+    check(pc.output, oracle(x), dtype)
+
+
+# ---------------------------------------------------------------- stage 2 alone
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,D", [(torch.float32, 64), (torch.bfloat16, 128), (torch.float16, 256), (torch.float32, 32)])
+def test_stage2_alone_merges_oracle_made_partials(dtype, D):
+    bsz, hq, hkv, L, tmax = 4, 6, 3, 5, 2048
+    lens = [2048, 700, 0, 1100]
+    x = make(72, bsz, hq, hkv, L, D, tmax, dtype, lens)
+    pc = prepare(x, _force_splits=6)
+    S = pc.plan.num_splits
+    chunk = pc.plan.chunk_for(max(lens))
+    s_of = [live_splits(t, chunk, S) for t in lens]
+    assert S >= 4 and s_of[0] == S and 1 < s_of[1] < S and s_of[2] == 1      # full, partly filled and one-slot sequences
+    g = torch.Generator().manual_seed(3)
+    mid_o = torch.randn(bsz, hq, S, L, D, generator=g)
+    mid_lse = torch.randn(bsz, hq, S, L, generator=g) * 3.0
+    # splits without an attendable key: lse -inf and a zero partial (what stage 1 writes for them)
+    dead = torch.rand(bsz, hq, S, L, generator=g) < 0.15
+    dead[0, 0, :, 0] = True                                                   # a row with no live split at all -> zeros
+    mid_lse[dead] = -math.inf
+    mid_o[dead] = 0.0
+    for b in range(bsz):                                                      # slots a sequence does not fill must not be read
+        mid_o[b, :, s_of[b]:] = float("nan")
+        mid_lse[b, :, s_of[b]:] = float("nan")
+    pc.mid_output.copy_(mid_o), pc.mid_output_lse.copy_(mid_lse)
+    pc.output.fill_(float("nan"))
+    pc.run_stage2()
+    torch.cuda.synchronize()
+    out = pc.output.float().cpu()
+    assert torch.isfinite(out).all()
+    for b in range(bsz):
+        ref, _ = stage2_merge_oracle([mid_o[b, :, s].double() for s in range(s_of[b])], [mid_lse[b, :, s].double() for s in range(s_of[b])])
+        torch.testing.assert_close(out[b].double(), ref, **TOL[dtype])
+    assert out[0, 0, 0].abs().max() == 0
+
+
+# ---------------------------------------------------------------- capacity far above the lengths
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [
+    # bsz hq hkv  L   D   tmax   dtype           lens
+    (4, 16, 4, 64, 128, 32768, torch.bfloat16, [2000, 1500, 64, 1999]),       # 256-row MFMA workgroups
+    (2, 8, 2, 16, 128, 65536, torch.float16, [3000, 10]),                     # 128-row MFMA workgroups
+    (1, 8, 8, 1, 128, 65536, torch.float16, [5000]),                          # plain decode
+    (2, 4, 4, 4, 64, 16384, torch.float32, [900, 901]),                       # shuffle kernel
+    (300, 2, 1, 4, 64, 4096, torch.bfloat16, None),                           # more sequences than the ordering pass takes
+])
+def test_cache_capacity_far_above_the_lengths(shape):
+    """No hint, a big cache: the result is the oracle's, equal (to rounding) with and without the hint,
+    and the plan spreads the live keys over the grid instead of leaving them in the first split."""
+    bsz, hq, hkv, L, D, tmax, dtype, lens = shape
+    if lens is None:
+        lens = [(37 * i) % 400 for i in range(bsz)]
+    x = make(73, bsz, hq, hkv, L, D, tmax, dtype, lens)
+    ref = oracle(x)
+    pc = prepare(x)
+    out = pc.run().clone()
+    check(out, ref, dtype)
+    hinted = prepare(x, max_seq_len_in_batch=max(lens))
+    check(hinted.run(), ref, dtype)
+    if pc.plan.num_splits > 1 and max(lens) >= 1024:
+        chunk = pc.plan.chunk_for(max(lens))
+        assert live_splits(max(lens), chunk, pc.plan.num_splits) >= min(pc.plan.num_splits, hinted.plan.num_splits, 2)
+
+
+@pytest.mark.gpu
+def test_paged_table_far_wider_than_the_sequences():
+    from test_parity_gpu import to_pages
+    x = make(74, 3, 8, 2, 64, 128, 1024, torch.bfloat16, [1000, 300, 0])
+    ref = oracle(x)
+    kp, vp, tables = to_pages(x, 64, seed=9)
+    wide_tables = torch.zeros(3, 512, dtype=torch.int32, device=DEV)      # room for 32768 positions per sequence
+    wide_tables[:, : tables.size(1)] = tables
+    xp = dict(x, k_cache=kp, v_cache=vp)
+    pc = prepare(xp, block_tables=wide_tables)
+    assert pc.args.cache_len == 512 * 64
+    check(pc.run(), ref, torch.bfloat16)
+
+
+# ---------------------------------------------------------------- the 64-row-wave loop
+WIDE_CASES = [
+    # name                              bsz hq hkv  L   D    T     lens                          splits dtype         scale_k hot
+    ("6 full tiles", 1, 4, 1, 64, 128, 384, [384], 1, torch.bfloat16, 1.0, None),
+    ("1 .. 12 full tiles", 9, 4, 1, 64, 128, 768, [64, 128, 192, 256, 320, 384, 448, 512, 768], 1, torch.bfloat16, 1.0, None),
+    ("ragged tails", 4, 4, 1, 64, 128, 1024, [777, 150, 37, 0], 1, torch.bfloat16, 1.0, None),
+    ("3 splits", 1, 4, 1, 64, 128, 2048, [2048], 3, torch.bfloat16, 1.0, None),
+    ("192 rows: one wave without rows", 1, 6, 1, 32, 128, 1024, [1000], 2, torch.bfloat16, 1.0, None),
+    ("160 rows of 16", 1, 10, 1, 16, 128, 768, [768], 1, torch.bfloat16, 1.0, None),
+    ("a late key raises every row maximum", 1, 4, 1, 64, 128, 1024, [1024], 1, torch.bfloat16, 1.0, 900),
+    ("fp16", 1, 4, 1, 64, 128, 1024, [1000], 2, torch.float16, 1.0, None),
+    ("fp16, late key", 1, 4, 1, 64, 128, 1024, [1024], 1, torch.float16, 1.0, 900),
+    ("head_dim 64", 1, 4, 1, 64, 64, 1024, [1000], 2, torch.bfloat16, 1.0, None),
+    ("head_dim 64, fp16, late key", 1, 8, 1, 32, 64, 1024, [1024], 1, torch.float16, 1.0, 700),
+    ("ragged batch", 5, 8, 2, 64, 128, 4096, [4096, 100, 2500, 64, 3333], 3, torch.bfloat16, 1.0, None),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", WIDE_CASES, ids=lambda c: c[0])
+def test_64_row_wave_loop_against_the_oracle(case):
+    """The hand-scheduled loop (4 waves x 64 rows, one K/V fragment read feeding two MFMAs): full tiles
+    run in the loop, the ragged tail and the tree block in its masked halves; a key that raises the row
+    maxima late in the stream forces the exact redo of the lazy softmax. Also against the 8-wave loop."""
+    name, bsz, hq, hkv, L, D, T, lens, splits, dtype, scale_k, hot = case
+    print("case:", name, flush=True)
+    x = make(75, bsz, hq, hkv, L, D, T, dtype, lens)
+    if scale_k != 1.0:
+        x["k_cache"] = (x["k_cache"].float() * scale_k).to(dtype)
+    if hot is not None:
+        x["k_cache"][:, :, hot, :] = (x["q"][:, :: hq // hkv, 0, :].float() * 3).to(dtype)
+    ref = oracle(x)
+    pc = prepare(x, _force_splits=splits, _force_kernel=_lib.KERNEL_MFMA_WIDE)
+    assert pc.plan.kernel == _lib.KERNEL_MFMA and pc.plan.rows_per_wg == 256 and pc.plan.mfma_loop == 1
+    out = pc.run().clone()
+    check(out, ref, dtype)
+    narrow = prepare(x, _force_splits=splits, _force_kernel=_lib.KERNEL_MFMA)
+    assert narrow.plan.mfma_loop == 0
+    torch.testing.assert_close(out.float(), narrow.run().float(), **TOL[dtype])
+    if pc.plan.counter_elems:
+        check(pc.run_single_launch(), ref, dtype)
+
+
+@pytest.mark.gpu
+def test_64_row_wave_loop_is_refused_where_it_does_not_exist():
+    x = make(76, 1, 4, 2, 8, 128, 256, torch.bfloat16, [256])                 # 16-row units
+    with pytest.raises(ValueError, match="status -9"):
+        prepare(x, _force_kernel=_lib.KERNEL_MFMA_WIDE)
+
+
+@pytest.mark.gpu
+def test_64_row_wave_loop_at_headline_size():
+    cfg = CONFIGS["cfg3_gqa_8b_bf16"]
+    x = make_inputs(cfg, seed=0, device=DEV, gen_device=DEV)
+    pc = prepare(x, _force_kernel=_lib.KERNEL_MFMA_WIDE)
+    assert pc.plan.mfma_loop == 1
+    check(pc.run(), oracle(x), cfg.dtype)
+
+
+# ---------------------------------------------------------------- head_dim 256: merge inside stage 1, paged caches
+@pytest.mark.gpu
+@pytest.mark.parametrize("splits", [2, 3])
+def test_head_dim_256_single_launch_and_paged(splits):
+    from test_parity_gpu import to_pages
+    x = make(77, 3, 8, 4, 40, 256, 900, torch.bfloat16, [900, 450, 1])       # 80 rows per unit
+    ref = oracle(x)
+    pc = prepare(x, _force_splits=splits)
+    assert pc.plan.kernel == _lib.KERNEL_MFMA and pc.plan.rows_per_wg == 128 and pc.plan.counter_elems > 0
+    two = pc.run_two_launches().clone()
+    check(two, ref, torch.bfloat16)
+    for _ in range(2):
+        pc.output.fill_(float("nan"))
+        one = pc.run_single_launch().clone()
+        check(one, ref, torch.bfloat16)
+        torch.testing.assert_close(one.float(), two.float(), atol=1e-5, rtol=2 ** -7)
+    kp, vp, tables = to_pages(x, 32, seed=1)
+    paged = prepare(dict(x, k_cache=kp, v_cache=vp), _force_splits=splits, block_tables=tables, max_seq_len_in_batch=900)
+    plain = prepare(x, _force_splits=splits, max_seq_len_in_batch=900)
+    out_paged = paged.run().clone()
+    check(out_paged, ref, torch.bfloat16)
+    assert torch.equal(out_paged, plain.run())
+
+
+# ---------------------------------------------------------------- the headline size against fp64 on the CPU
+@pytest.mark.gpu
+def test_headline_sequence_against_the_fp64_oracle_on_the_cpu():
+    """One sequence and two query heads (the first head of the first cache head, the last head of the
+    last) of the headline workload, checked against the oracle in float64 on the CPU: the GPU's own
+    matmuls take no part in the expected values."""
+    cfg = CONFIGS["cfg3_gqa_8b_bf16"]
+    x = make_inputs(cfg, seed=0, device=DEV, gen_device=DEV)
+    out = prepare(x).run()
+    b, heads = 3, [0, cfg.num_heads - 1]
+    kv_heads = [h // cfg.kv_group_num for h in heads]
+    cpu = lambda t: t.cpu()
+    ref = tree_attention_oracle(cpu(x["q"][b:b + 1, heads]), cpu(x["k_cache"][b:b + 1, kv_heads]), cpu(x["v_cache"][b:b + 1, kv_heads]),
+                                cpu(x["current_k"][b:b + 1, kv_heads]), cpu(x["current_v"][b:b + 1, kv_heads]), cpu(x["mask"]),
+                                cpu(x["kv_seq_len"][b:b + 1]), x["sm_scale"], 1, dtype=torch.float64)
+    assert ref.device.type == "cpu" and ref.dtype == torch.float64
+    torch.testing.assert_close(out[b:b + 1, heads].cpu().double(), ref, **TOL[cfg.dtype])
+
+
+# ---------------------------------------------------------------- how much of the tolerance is used
+# Largest |out - ref| / (atol + rtol |ref|) a configuration may reach: half the tolerance. A change that
+# trades precision for speed (fp16 partials, cheaper exponentials) has to fit under it or move it knowingly.
+MARGIN = 0.5
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["cfg1_plumbing_fp32", "cfg2_medusa_7b_fp16", "cfg3_gqa_8b_bf16", "cfg4_long_ctx_bf16", "cfg5_ragged_70b_bf16"])
+def test_error_margin_of_the_benchmark_configurations(name):
+    cfg = CONFIGS[name]
+    big = cfg.bsz * cfg.cache_len > (1 << 16)
+    x = make_inputs(cfg, seed=0, device=DEV, gen_device=DEV if big else "cpu")
+    ref = oracle(x).float()
+    out = prepare(x).run().float()
+    err = (out - ref).abs()
+    tol = TOL[cfg.dtype]
+    share = (err / (tol["atol"] + tol["rtol"] * ref.abs())).max().item()
+    rel = (err / ref.abs().clamp_min(1e-6))[ref.abs() > 1e-2]
+    print(f"\n{name}: max abs err {err.max().item():.3e}, max rel err (|ref| > 1e-2) {rel.max().item() if rel.numel() else 0.0:.3e}, "
+          f"largest share of the tolerance {share:.3f}", flush=True)
+    assert share <= MARGIN, (name, share)
