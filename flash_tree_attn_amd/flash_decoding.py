@@ -8,8 +8,10 @@ Differences from the reference that a caller can observe (all deliberate):
   (flash_tree_attn.py:373-376).
 * `mid_output` / `mid_output_lse` are scratch for at most `plan.num_splits` splits
   (never more than ceil(max_len / block_size), so reference-sized buffers fit).
-* No host sync: `kv_seq_len.max().item()` (flash_tree_attn.py:272) is not needed;
-  `max_seq_len_in_batch` is only a hint that shrinks the grid.
+* No host sync: `kv_seq_len.max().item()` (flash_tree_attn.py:272) is not needed.
+  `max_seq_len_in_batch` (any upper bound of the lengths) or, without it, the cache
+  capacity bounds the grid and the scratch; how the keys are cut into chunks follows
+  the real lengths, which the kernels read themselves.
 * fp16, bf16 and fp32 inputs; `current_k/current_v` with num_kv_heads or num_heads
   heads; any q_len >= 1; `mask` float (additive, flash_tree_attn.py:368), bool, or int64
   bit words from `tree_mask.pack_mask` (8 bytes per row and 64 tree keys).
@@ -35,21 +37,37 @@ class FtaAssertionError(ValueError, AssertionError):
 
 _ASSERT_STATUSES = {-2, -3, -4, -5}
 _cu_count = {}
-_counters = {}
+_counters = {}           # (device index, stream handle) -> the int32 counter buffer calls on that stream use
+_retired_counters = []   # buffers a larger one replaced: kept alive, an earlier launch or a captured graph may still name them
+_suspect_counters = set()   # keys whose last launch returned an error: cleared before the next use
 
 
 def _counters_for(device: torch.device, stream: int, elems: int) -> Optional[torch.Tensor]:
-    """Zeroed int32 counters for the single-launch merge. The kernel leaves them zero
-    again, so one buffer per (device, stream) serves every call issued on that stream;
-    calls on different streams may overlap in time and get buffers of their own."""
+    """Zeroed int32 counters for the single-launch merge, or None where the call has to take two
+    launches. The kernel leaves the counters zero again, so one buffer per (device, stream)
+    serves every call issued on that stream; calls on different streams may overlap in time and
+    get buffers of their own. A buffer, once handed out, lives until the process ends. While
+    the stream is capturing a graph the answer is None: a graph would keep the buffer's
+    address for as long as it is replayed, next to eager calls that count in the same memory."""
+    if torch.cuda.is_current_stream_capturing():
+        return None
     key = (device.index, stream)
     buf = _counters.get(key)
     if buf is None or buf.numel() < elems:
-        if torch.cuda.is_current_stream_capturing():
-            return None   # no allocation and fill inside a captured graph: the call takes two launches there
+        if buf is not None:
+            _retired_counters.append(buf)
         buf = torch.zeros(max(elems, 4096), dtype=torch.int32, device=device)
         _counters[key] = buf
+        _suspect_counters.discard(key)
+    elif key in _suspect_counters:
+        buf.zero_()   # a launch that failed may have left counts behind: every later merge would wait for ever-missing partials
+        _suspect_counters.discard(key)
     return buf
+
+
+def _launch_failed(device: torch.device, stream: int) -> None:
+    if (device.index, stream) in _counters:
+        _suspect_counters.add((device.index, stream))
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
@@ -227,6 +245,8 @@ class PreparedCall:
             self.args.counters, self.args.counter_elems = None, 0
         status = fn(self._ref, stream)
         if status:
+            if buf is not None:
+                _launch_failed(self._device, stream)
             _check(status)
         return self.output
 
@@ -260,6 +280,18 @@ def prepare(q, k_cache, v_cache, current_k, current_v, mask, kv_seq_len, block_s
                             max_seq_len_in_batch, sm_scale, kv_group_num, _force_splits, _force_kernel, block_tables)
     bsz, hq, L, D = q.shape
     dev = q.device
+    # scratch the caller brought is known to the plan: it bounds the split count the heuristic may pick
+    user_mid = mid_output is not None and mid_output_lse is not None
+    for name, t, nd in (("mid_output", mid_output, 5), ("mid_output_lse", mid_output_lse, 4)):
+        if t is None:
+            continue
+        if t.dim() != nd or t.dtype != torch.float32 or t.device != dev or t.stride(-1) != 1:
+            raise FtaAssertionError(f"{name} must be a float32 tensor with {nd} dims on q's device")
+        if t.size(0) < bsz or t.size(1) != hq or t.size(3) != L or (nd == 5 and t.size(4) != D):
+            raise FtaAssertionError(f"{name} has incompatible shape {tuple(t.shape)}")
+    if user_mid:
+        args.mid_o, args.mid_lse = mid_output.data_ptr(), mid_output_lse.data_ptr()
+        args.mid_splits = min(mid_output.size(2), mid_output_lse.size(2))
     pl = plan_for(args, _num_cus(dev))
 
     if output is None:
@@ -277,13 +309,6 @@ def prepare(q, k_cache, v_cache, current_k, current_v, mask, kv_seq_len, block_s
             mid_output = torch.empty((bsz, hq, pl.num_splits, L, D), dtype=torch.float32, device=dev)
         if mid_output_lse is None:
             mid_output_lse = torch.empty((bsz, hq, pl.num_splits, L), dtype=torch.float32, device=dev)
-        for name, t, nd in (("mid_output", mid_output, 5), ("mid_output_lse", mid_output_lse, 4)):
-            if t.dim() != nd or t.dtype != torch.float32 or t.device != dev or t.stride(-1) != 1:
-                raise FtaAssertionError(f"{name} must be a float32 tensor with {nd} dims on q's device")
-            if t.size(0) < bsz or t.size(1) != hq or t.size(3) != L:
-                raise FtaAssertionError(f"{name} has incompatible shape {tuple(t.shape)}")
-        if mid_output.size(4) != D:
-            raise FtaAssertionError(f"mid_output has incompatible shape {tuple(mid_output.shape)}")
         args.mid_o, args.mid_lse = mid_output.data_ptr(), mid_output_lse.data_ptr()
         args.mid_splits = min(mid_output.size(2), mid_output_lse.size(2))
         args.mid_o_stride[:] = mid_output.stride()[:4]
@@ -372,6 +397,8 @@ def _run_remembered(e, q, k_cache, v_cache, current_k, current_v, mask, kv_seq_l
         a.counters, a.counter_elems = None, 0
     status = e.decode(e.ref, stream)
     if status:
+        if buf is not None:
+            _launch_failed(e.device, stream)
         _check(status)
     return output
 

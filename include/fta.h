@@ -86,7 +86,14 @@ typedef enum fta_kernel {
  *             between the two launches. Contract: all zero on entry; the kernel leaves
  *             them all zero again, so one buffer zeroed once serves every later call on
  *             the same stream; calls that may overlap in time need buffers of their
- *             own. NULL keeps the two-launch path.
+ *             own. A launch that fails, or a kernel that does not run to its end (a
+ *             device fault, a reset), may leave counts behind: zero the buffer again
+ *             before its next use, or no workgroup of a later call ever sees the last
+ *             arrival and `out` stays unwritten, without an error. The buffer must stay
+ *             allocated until every launch that was given it has finished; a captured
+ *             graph holds its address for as long as the graph is replayed, and replays
+ *             must not overlap eager calls on the same buffer. NULL keeps the two-launch
+ *             path.
  */
 typedef struct fta_args {
   const void* q;

@@ -338,3 +338,24 @@ def test_split_heuristic_against_measured_sweeps(fta_lib):
     assert len(uniform) == 112 and len(ragged) == 76
     assert sum(uniform) / len(uniform) < 1.05 and max(uniform) < 1.35
     assert sum(ragged) / len(ragged) < 1.06 and max(ragged) < 1.40
+
+
+def test_scratch_the_caller_brought_bounds_the_split_count(fta_lib):
+    """A caller of the reference sizes mid_output from the batch's longest sequence
+    (flash_tree_attn.py:274-281) and may pass no length bound: the plan, cut for the cache
+    capacity, must then stay within those slots instead of asking for more."""
+    big = dict(bsz=1, cache_len=131072, v_cache_len=131072)
+    st, free = plan(fta_lib, base_args(**big))
+    assert st == 0 and free.num_splits > 8
+    a = base_args(**big)
+    a.mid_o = a.mid_lse = 0x1000
+    a.mid_splits = 8
+    st, pl = plan(fta_lib, a)
+    assert st == 0 and 1 < pl.num_splits <= 8 and pl.num_splits * pl.chunk >= 131072
+    assert all(-(-b // c) <= pl.num_splits for b, c in zip(pl.len_bound, pl.chunk_by_len))
+    a.mid_splits = 1
+    st, pl = plan(fta_lib, a)
+    assert st == 0 and pl.num_splits == 1
+    a.force_splits = 4                      # a pinned count is the caller's word: it is planned, and fta_decode refuses the scratch
+    st, pl = plan(fta_lib, a)
+    assert st == 0 and pl.num_splits == 4

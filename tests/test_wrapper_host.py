@@ -90,3 +90,39 @@ def test_misaligned_contiguous_tensor_is_cloned():
     assert r.data_ptr() % 16 == 0 and torch.equal(r, t)
     ok = torch.zeros(4, 64, dtype=torch.float16)
     assert fd._as_rows(ok) is ok
+
+
+def test_counter_buffers_are_never_dropped_and_are_cleared_after_a_failed_launch(monkeypatch):
+    """The single-launch merge counts arrivals in a buffer the wrapper keeps per (device, stream).
+    An earlier launch may still be running on a buffer when a larger one replaces it, so replaced
+    buffers stay alive; a capturing stream gets none (the graph would keep its address); a launch
+    that returned an error may have left counts behind, so the buffer is cleared before its next use."""
+    capturing = [False]
+    monkeypatch.setattr(torch.cuda, "is_current_stream_capturing", lambda: capturing[0])
+    monkeypatch.setattr(fd, "_counters", {})
+    monkeypatch.setattr(fd, "_retired_counters", [])
+    monkeypatch.setattr(fd, "_suspect_counters", set())
+    dev = torch.device("cpu")
+    a = fd._counters_for(dev, 7, 100)
+    assert a.dtype == torch.int32 and a.numel() >= 100 and int(a.abs().sum()) == 0
+    assert fd._counters_for(dev, 7, 50) is a                       # reused while it is large enough
+    other = fd._counters_for(dev, 8, 50)
+    assert other is not a                                          # a buffer per stream
+    big = fd._counters_for(dev, 7, a.numel() + 1)
+    assert big is not a and big.numel() > a.numel()
+    assert any(r is a for r in fd._retired_counters)               # the replaced one is kept alive
+    assert fd._counters[(None, 7)] is big
+
+    capturing[0] = True
+    assert fd._counters_for(dev, 7, 10) is None                    # even though this stream has a buffer
+    assert fd._counters_for(dev, 9, 10) is None and (None, 9) not in fd._counters
+    capturing[0] = False
+
+    big[:5] = 3                                                    # what a launch that died half-way leaves behind
+    fd._launch_failed(dev, 7)
+    again = fd._counters_for(dev, 7, 10)
+    assert again is big and int(big.abs().sum()) == 0
+    big[0] = 1                                                     # not suspect any more: the wrapper does not touch it
+    assert fd._counters_for(dev, 7, 10) is big and int(big[0]) == 1
+    fd._launch_failed(dev, 12345)                                  # a stream without a buffer: nothing to remember
+    assert (None, 12345) not in fd._suspect_counters
