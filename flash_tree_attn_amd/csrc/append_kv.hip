@@ -133,11 +133,7 @@ extern "C" int fta_append_kv(const fta_append_args* args, void* hip_stream) {
   const int64_t threads = std::max<int64_t>(static_cast<int64_t>(a.bsz) * a.max_accept * a.num_kv_heads * 2 * (p.row_bytes / 16), a.bsz);
   const int64_t grid = (threads + 255) / 256;
   if (grid > 0x7fffffffLL) return FTA_ERR_SHAPE;
-  hipLaunchKernelGGL(append_kv_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, p);
-  if (hipGetLastError() != hipSuccess) return FTA_ERR_LAUNCH;
-  if (in_place) {
-    hipLaunchKernelGGL(append_len_kernel, dim3((a.bsz + 255) / 256), dim3(256), 0, stream, p);
-    if (hipGetLastError() != hipSuccess) return FTA_ERR_LAUNCH;
-  }
+  if (int st = fta::launch_checked(append_kv_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, p)) return st;
+  if (in_place) return fta::launch_checked(append_len_kernel, dim3((a.bsz + 255) / 256), dim3(256), 0, stream, p);
   return FTA_OK;
 }

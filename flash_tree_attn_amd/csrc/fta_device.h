@@ -21,6 +21,14 @@ typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
 
 #define FTA_LDS __attribute__((address_space(3)))
 
+// Launches `kern(params)` and reports what THIS launch returned (the thread's sticky last-error
+// state may hold an older, unrelated failure and is neither read nor cleared).
+template <typename Kernel, typename Params>
+inline int launch_checked(Kernel kern, dim3 grid, dim3 block, unsigned smem_bytes, hipStream_t stream, const Params& params) {
+  void* args[] = {const_cast<Params*>(&params)};
+  return hipLaunchKernel(reinterpret_cast<const void*>(kern), grid, block, args, smem_bytes, stream) == hipSuccess ? FTA_OK : FTA_ERR_LAUNCH;
+}
+
 __device__ __forceinline__ float neg_inf() { return -__builtin_huge_valf(); }
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }

@@ -217,8 +217,7 @@ int launch(const KernelParams& p, hipStream_t stream) {
   }
   const int64_t grid = static_cast<int64_t>(p.bsz) * p.units * p.row_blocks * p.num_splits;
   if (grid <= 0 || grid > 0x7fffffffLL) return FTA_ERR_SHAPE;
-  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(grid)), dim3(256), S::kTotal, stream, p);
-  return hipGetLastError() == hipSuccess ? FTA_OK : FTA_ERR_LAUNCH;
+  return launch_checked(kern, dim3(static_cast<unsigned>(grid)), dim3(256), S::kTotal, stream, p);
 }
 
 template <typename T>

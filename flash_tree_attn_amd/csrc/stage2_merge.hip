@@ -70,8 +70,7 @@ int launch(const KernelParams& p, hipStream_t stream) {
   const int64_t total_rows = static_cast<int64_t>(p.bsz) * p.num_q_heads * p.q_len;
   const int64_t grid = (total_rows + kRowsPerBlock - 1) / kRowsPerBlock;
   if (grid <= 0 || grid > 0x7fffffffLL) return FTA_ERR_SHAPE;
-  hipLaunchKernelGGL((stage2_merge_kernel<T, D>), dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, p);
-  return hipGetLastError() == hipSuccess ? FTA_OK : FTA_ERR_LAUNCH;
+  return launch_checked(stage2_merge_kernel<T, D>, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, p);
 }
 
 template <typename T>
