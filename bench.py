@@ -335,7 +335,7 @@ def main():
                    "head_dim": cfg.head_dim, "q_len": cfg.q_len, "cache_len": cfg.cache_len, "lengths": cfg.lengths,
                    "block_size": cfg.block_size, "mask": "packed u64" if args.packed_mask else "additive f32",
                    "kv_layout": f"paged, {args.paged} positions per page, shuffled pool" if args.paged else "contiguous per sequence", "kv_sets_rotated": kv_sets, "num_splits": plan.num_splits,
-                   "chunk": plan.chunk, "stage1_kernel": ("mfma_wide" if plan.mfma_loop else "mfma") if plan.kernel == _lib.KERNEL_MFMA else "shuffle",
+                   "chunk": plan.chunk, "chunk_for_these_lengths": plan.chunk_for(int(x["kv_seq_len"].max())), "stage1_kernel": ("mfma_wide" if plan.mfma_loop else "mfma") if plan.kernel == _lib.KERNEL_MFMA else "shuffle",
                    "stage1_workgroups": plan.num_workgroups, "algorithmic_bytes": nbytes, "flops": nflops},
         "tflops": nflops / (ms * 1e-3) / 1e12,
         "roofline": {"bound": "hbm", "kernel": "stage1", "achieved": round(gbs_s1, 1), "peak": HBM_PEAK_GBS,
