@@ -83,6 +83,64 @@ def test_no_hand_issued_load_into_registers(kernels):
                     assert "sc1" in l, (name, l)
 
 
+REG = re.compile(r"\b([va])(\d+)\b|\b([va])\[(\d+):(\d+)\]")
+
+
+def vector_regs(text):
+    out = set()
+    for m in REG.finditer(text):
+        if m.group(1):
+            out.add((m.group(1), int(m.group(2))))
+        else:
+            out.update((m.group(3), i) for i in range(int(m.group(4)), int(m.group(5)) + 1))
+    return out
+
+
+def touches_of_in_flight_lds_reads(ins):
+    """Operand fragments are read with hand-written `ds_read` instructions and awaited by separate hand-written
+    `s_waitcnt lgkmcnt(n)`: between the two the compiler believes the destination holds its value. Walks one
+    kernel in layout order, keeps the destinations of the hand-issued reads that no wait has covered yet (LDS
+    reads return in order, a wait for n leaves the newest n in flight) and reports every instruction that
+    names such a register. Returns (problems, reads seen)."""
+    in_asm, pending, problems, reads = False, [], [], 0
+    for idx, l in enumerate(ins):
+        if l.startswith(";;#ASMSTART"):
+            in_asm = True
+            continue
+        if l.startswith(";;#ASMEND"):
+            in_asm = False
+            continue
+        op = l.split()[0]
+        if op == "s_waitcnt":
+            m = re.search(r"lgkmcnt\((\d+)\)", l)
+            if m:
+                pending = pending[len(pending) - int(m.group(1)):] if int(m.group(1)) else []
+            continue
+        live = set().union(*pending) if pending else set()
+        if in_asm and op.startswith("ds_read"):
+            reads += 1
+            dest = vector_regs(l.split(",")[0])
+            if dest & live:
+                problems.append((idx, l))
+            pending.append(dest)
+        elif vector_regs(l) & live:
+            problems.append((idx, l))
+    return problems, reads
+
+
+def test_registers_of_in_flight_lds_reads_are_left_alone(kernels):
+    for name, (ins, _) in kernels.items():
+        problems, reads = touches_of_in_flight_lds_reads(ins)
+        assert reads >= 32, (name, reads)            # every variant reads its K and V fragments this way
+        assert not problems, (name, problems[:3])
+    # the check sees what it is meant to see: a copy of a destination right behind its read is reported
+    name, (ins, _) = next(iter(kernels.items()))
+    at = next(i for i, l in enumerate(ins) if l.startswith("ds_read") and ins[i - 1].startswith(";;#ASMSTART"))
+    first = sorted(vector_regs(ins[at].split(",")[0]))[0]
+    spoiled = ins[:at + 2] + [f"v_mov_b32 v255, {first[0]}{first[1]}"] + ins[at + 2:]
+    assert touches_of_in_flight_lds_reads(spoiled)[0]
+
+
 def test_the_whole_tile_pipelined_loop_has_no_spill_traffic(kernels):
     """Scratch accesses are vector-memory instructions too: inside the fused loop of the 8-wave
     kernels they would sit between the tile requests and the hand-counted waits and make every
