@@ -586,6 +586,100 @@ def verify(body: list[str], ops: str, name: str) -> None:
                     raise AssertionError(f"{name}: `{line}` reads undeclared {k}{sorted(bad)}")
 
 
+def hazards(body: list[str], name: str) -> None:
+    """Raises if the text breaks one of the issue rules the hardware does not enforce itself (the assembler inserts
+    nothing, and each of these showed up as wrong numbers on the GPU, never as a fault). Distances are in wait
+    states: every instruction counts one, `s_nop n` counts n + 1. Checked in layout order.
+      * the result of `v_dot2c` read by a different vector instruction: 3 wait states;
+      * the result of a transcendental (`v_exp_f32`) read by a vector instruction: 1;
+      * a write of M0 before the `global_load_lds` that uses it: 1;
+      * a VGPR result of an 8-pass MFMA touched by a non-MFMA instruction: 11;
+      * SCC: an `s_cselect` / `s_cbranch_scc` takes the compare before it, so nothing that writes SCC (`s_add`,
+        `s_addc`, ...) may stand between them; an `s_addc` takes the carry of the `s_add_u32` before it;
+      * the statement ends on at least 11 wait states without an MFMA (the compiler reads the accumulators next and
+        does not know the statement holds MFMAs)."""
+    import re
+    reg = re.compile(r"\b([vas])(\d+)\b|\b([vas])\[(\d+):(\d+)\]")
+
+    def regs(tok):
+        out = set()
+        for m in reg.finditer(tok):
+            if m.group(1):
+                out.add((m.group(1), int(m.group(2))))
+            else:
+                out.update((m.group(3), i) for i in range(int(m.group(4)), int(m.group(5)) + 1))
+        return out
+
+    ins = []
+    for line in body:
+        line = line.split(";")[0].strip()
+        if not line or line.endswith(":"):
+            continue
+        parts = line.split(None, 1)
+        ins.append((parts[0], [a.strip() for a in parts[1].split(",")] if len(parts) > 1 else [], line))
+
+    def dst_src(op, args):
+        every = set().union(*[regs(a) for a in args]) if args else set()
+        if op.startswith(("s_cmp", "s_cbranch", "s_branch", "s_waitcnt", "s_nop", "s_barrier", "global_load_lds")):
+            return set(), every
+        if op.startswith("v_cmp"):
+            return set(), set().union(*[regs(a) for a in args[1:]])
+        d = regs(args[0]) if args else set()
+        src = set().union(*[regs(a) for a in args[1:]]) if len(args) > 1 else set()
+        if op.startswith(("v_dot2c", "v_permlane32_swap")):
+            src |= d
+        if op.startswith("v_permlane32_swap"):
+            d |= regs(args[1])
+        return d, src
+
+    def wait_states(op, args):
+        return int(args[0]) + 1 if op == "s_nop" else 1
+
+    def too_close(i, need, offends):
+        dist = 0
+        for j in range(i + 1, len(ins)):
+            op, args, text = ins[j]
+            if offends(op, args):
+                raise AssertionError(f"{name}: `{text}` follows `{ins[i][2]}` after {dist} wait states, needs {need}")
+            dist += wait_states(op, args)
+            if dist >= need:
+                return
+
+    scc_writers = ("s_add", "s_sub", "s_and_b", "s_or_b", "s_xor", "s_lshl", "s_lshr", "s_ashr", "s_andn2", "s_orn2", "s_min", "s_max", "s_abs", "s_bfe")
+    for i, (op, args, text) in enumerate(ins):
+        d, _ = dst_src(op, args)
+        if op.startswith("v_dot2c"):
+            too_close(i, 3, lambda o, a: o.startswith("v_") and not o.startswith("v_dot2c") and dst_src(o, a)[1] & d)
+        if op.startswith(("v_exp_f32", "v_log_f32", "v_rcp_f32", "v_rsq_f32", "v_sqrt_f32")):
+            too_close(i, 1, lambda o, a: o.startswith("v_") and dst_src(o, a)[1] & d)
+        if op == "s_mov_b32" and args[0] == "m0":
+            too_close(i, 1, lambda o, a: o.startswith("global_load_lds"))
+        if op.startswith("v_mfma"):
+            vd = {r for r in d if r[0] == "v"}
+            if vd:
+                too_close(i, 11, lambda o, a: not o.startswith(("v_mfma", "s_")) and (dst_src(o, a)[0] | dst_src(o, a)[1]) & vd)
+        if op.startswith(("s_cselect", "s_cbranch_scc", "s_addc")):
+            for j in range(i - 1, -1, -1):
+                o = ins[j][0]
+                if o.startswith("s_cmp"):
+                    if op.startswith("s_addc"):
+                        raise AssertionError(f"{name}: `{text}` takes its carry from `{ins[j][2]}`")
+                    break
+                if o.startswith(scc_writers):
+                    if not (op.startswith("s_addc") and o.startswith("s_add_u32")):
+                        raise AssertionError(f"{name}: `{ins[j][2]}` overwrites SCC before `{text}`")
+                    break
+            else:
+                raise AssertionError(f"{name}: nothing sets SCC before `{text}`")
+    tail = 0
+    for op, args, text in reversed(ins):
+        if op.startswith("v_mfma") or op.startswith(("s_branch", "s_cbranch")):
+            break
+        tail += wait_states(op, args)
+    if tail < 11:
+        raise AssertionError(f"{name}: the statement ends {tail} wait states after an MFMA or a branch, needs 11")
+
+
 def render() -> str:
     lines = ["// Generated by gen_wide_loop.py - do not edit; edit the generator and run it.", "// clang-format off"]
     for D in (128, 64):
@@ -593,6 +687,7 @@ def render() -> str:
         for dtype in ("bf16", "f16"):
             body = gen(D, dtype)
             verify(body, operands(D), f"loop {D} {dtype}")
+            hazards(body, f"loop {D} {dtype}")
             lines.append(f"#define FTA_WIDE_LOOP_{D}_{dtype.upper()}() asm volatile( \\")
             for ins in body:
                 lines.append(f'      "{ins}\\n\\t" \\')
@@ -601,6 +696,7 @@ def render() -> str:
                 lines.append(f"#define FTA_WIDE_MASKED_{D}_{dtype.upper()}_H{H}() asm volatile( \\")
                 mbody = gen_masked(D, dtype, H)
                 verify(mbody, operands_masked(D), f"masked {D} {dtype} H{H}")
+                hazards(mbody, f"masked {D} {dtype} H{H}")
                 for ins in mbody:
                     lines.append(f'      "{ins}\\n\\t" \\')
                 lines.append(operands_masked(D).replace("\n", " \\\n") + ")")

@@ -218,3 +218,41 @@ def test_generator_rejects_undeclared_registers():
         gen.verify(gen.gen_masked(64, "f16", H), gen.operands_masked(64), "masked")
         with pytest.raises(AssertionError, match="undeclared"):
             gen.verify(gen.gen_masked(64, "f16", H), gen.operands_masked(64).replace(f'"v{gen.V_R}", ', ""), "masked, clobber dropped")
+
+
+def test_generator_rejects_issue_hazards():
+    """The rules the hardware does not enforce (wait states behind v_dot2c, transcendentals, M0 writes and MFMA
+    results; SCC between a compare and its consumer; the fence at the end of a statement): the rendered text
+    passes, and each rule fires on a text that breaks it."""
+    gen = _generator()
+    body = gen.gen(128, "bf16")
+    for D in (64, 128):
+        for dtype in ("bf16", "f16"):
+            gen.hazards(gen.gen(D, dtype), "loop")
+            for H in (0, 1):
+                gen.hazards(gen.gen_masked(D, dtype, H), "masked")
+
+    def first(pred):
+        return next(i for i, l in enumerate(body) if pred(l))
+
+    broken = list(body)
+    broken.pop(first(lambda l: l.startswith("s_nop 3")))                      # the gap behind a group of v_dot2c
+    with pytest.raises(AssertionError, match="v_dot2c.*needs 3"):
+        gen.hazards(broken, "dot")
+    at = first(lambda l: l.startswith("v_exp_f32"))
+    dest = body[at].split()[1].rstrip(",")
+    with pytest.raises(AssertionError, match="v_exp_f32.*needs 1"):
+        gen.hazards(body[:at + 1] + [f"v_add_f32 v{gen.V_T}, {dest}, {dest}"] + body[at + 1:], "trans")
+    at = first(lambda l: l.startswith("s_cselect"))
+    with pytest.raises(AssertionError, match="overwrites SCC"):
+        gen.hazards(body[:at] + [f"s_add_u32 s{gen.S_TMP}, s{gen.S_TMP}, 1"] + body[at:], "scc")
+    at = first(lambda l: l.startswith("v_mfma") and l.split()[1].startswith("v["))
+    with pytest.raises(AssertionError, match="needs 11"):
+        gen.hazards(body[:at + 1] + [f"v_add_f32 v{gen.V_T}, v{gen.V_S}, v{gen.V_S}"] + body[at + 1:], "mfma result")
+    at = first(lambda l: l.startswith("s_mov_b32 m0"))
+    assert body[at + 1].startswith("s_nop")
+    with pytest.raises(AssertionError, match="m0.*needs 1"):
+        gen.hazards(body[:at + 1] + body[at + 2:], "m0")
+    end = max(i for i, l in enumerate(body) if l.startswith("s_nop 15"))
+    with pytest.raises(AssertionError, match="statement ends"):
+        gen.hazards(body[:end] + ["s_nop 3"] + body[end + 1:], "fence")
