@@ -20,6 +20,11 @@ typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
 
 #define FTA_LDS __attribute__((address_space(3)))
+// The workgroup's dynamically sized LDS, as `char name[]`. A macro so that a test harness which runs these
+// kernels on host threads can put an ordinary buffer there.
+#ifndef FTA_DYNAMIC_LDS
+#define FTA_DYNAMIC_LDS(name) extern __shared__ __attribute__((aligned(16))) char name[]
+#endif
 
 // Launches `kern(params)` and reports what THIS launch returned (the thread's sticky last-error
 // state may hold an older, unrelated failure and is neither read nor cleared).

@@ -228,7 +228,7 @@ stage1_mfma_kernel(const KernelParams p) {
   constexpr int kRowsPerWg = NW * kRowsPerWave;
   constexpr int kVRing = NSK * TL::kTileBytes;       // byte offset of the V ring
 
-  extern __shared__ __attribute__((aligned(16))) char smem[];
+  FTA_DYNAMIC_LDS(smem);
 
   const WorkItem w = decode_work(p, blockIdx.x);
   int b, split, T_b, chunk;   // chunk: keys per split of this launch, from the batch's longest sequence

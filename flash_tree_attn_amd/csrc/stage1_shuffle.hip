@@ -34,7 +34,7 @@ __global__ void __launch_bounds__(256) stage1_shuffle_kernel(const KernelParams 
   using S = ShuffleSmem<T, D>;
   constexpr int kVec = S::kVec;
   constexpr int kNC = D >= 64 ? D / 64 : 1;  // head_dim columns per lane in P.V
-  extern __shared__ __attribute__((aligned(16))) char smem[];
+  FTA_DYNAMIC_LDS(smem);
   T* Ks = reinterpret_cast<T*>(smem);
   T* Vs = reinterpret_cast<T*>(smem + S::kKBytes);
   float* Qs = reinterpret_cast<float*>(smem + S::kKBytes + S::kVBytes);

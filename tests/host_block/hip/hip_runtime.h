@@ -1,12 +1,18 @@
-// Host stand-in for the few HIP names that fta_device.h uses, so that its device functions (the
-// dispatch order, the chunk choice, the block-wide reductions) can run on the CPU exactly as written:
-// one host thread per GPU thread, std::barrier for __syncthreads, an exchange array per wave for
-// __shfl_xor. Test infrastructure only; one block runs at a time (so `__shared__` is a plain static).
+// Host stand-in for the HIP names that the simpler kernels of this library use, so that their source
+// runs on the CPU exactly as written: one host thread per GPU thread, std::barrier for __syncthreads,
+// an exchange array per wave for __shfl_xor, a plain buffer for the dynamic LDS, and hipLaunchKernel
+// = "run the grid, one workgroup after the other". TEST INFRASTRUCTURE ONLY: nothing under
+// flash_tree_attn_amd/ includes or loads this; it exists so that device code can be checked against the
+// oracle where no GPU is at hand (tests/test_dispatch_host.py, tests/test_host_block_kernels.py). Kernels
+// that use matrix instructions or inline assembly cannot run here. One workgroup runs at a time, so
+// `__shared__` is a plain static.
 #pragma once
 #include <algorithm>
 #include <barrier>
 #include <cmath>
 #include <cstdint>
+#include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <memory>
 #include <stdexcept>
@@ -26,9 +32,14 @@ struct dim3 {
 };
 typedef void* hipStream_t;
 enum hipError_t { hipSuccess = 0, hipErrorUnknown = 1 };
-inline hipError_t hipLaunchKernel(const void*, dim3, dim3, void**, unsigned, hipStream_t) { return hipErrorUnknown; }
+enum hipDeviceAttribute_t { hipDeviceAttributeMultiprocessorCount };
+enum hipFuncAttribute { hipFuncAttributeMaxDynamicSharedMemorySize };
+inline hipError_t hipGetDevice(int* dev) { *dev = 0; return hipSuccess; }
+inline hipError_t hipDeviceGetAttribute(int* value, hipDeviceAttribute_t, int) { *value = 256; return hipSuccess; }
+inline hipError_t hipFuncSetAttribute(const void*, hipFuncAttribute, int) { return hipSuccess; }
 
 namespace host_block {
+constexpr size_t kLdsBytes = 160 * 1024;
 struct Block {
   unsigned threads;
   std::barrier<> all;
@@ -39,12 +50,15 @@ struct Block {
   }
 };
 inline Block*& current() { static Block* b = nullptr; return b; }
+inline char* dynamic_lds() { alignas(16) static char lds[kLdsBytes]; return lds; }
 }  // namespace host_block
+#define FTA_DYNAMIC_LDS(name) char* name = host_block::dynamic_lds()
 
 inline thread_local dim3 threadIdx, blockIdx;
 inline dim3 blockDim, gridDim;
 
 inline void __syncthreads() { host_block::current()->all.arrive_and_wait(); }
+inline void host_wave_barrier() { host_block::current()->wave[threadIdx.x / 64]->arrive_and_wait(); }
 
 template <typename T>
 inline T __shfl_xor(T v, int mask, int /*width*/) {
@@ -63,11 +77,48 @@ inline T __shfl_xor(T v, int mask, int /*width*/) {
 // and the stand-in holds them to that.
 inline int host_readfirstlane(int v) {
   const int first = __shfl_xor(v, static_cast<int>(threadIdx.x & 63), 64);   // lane ^ lane = lane 0
-  if (first != v) throw std::logic_error("readfirstlane on a value that differs between lanes");
+  if (first != v) {
+    std::fprintf(stderr, "readfirstlane on a value that differs between lanes\n");
+    std::abort();
+  }
   return first;
 }
 #define __builtin_amdgcn_readfirstlane(x) host_readfirstlane(x)
 #define __builtin_amdgcn_exp2f(x) exp2f(x)
 #define __builtin_amdgcn_logf(x) log2f(x)
+#define __builtin_amdgcn_fence(order, scope) ((void)0)
+#define __builtin_amdgcn_wave_barrier() host_wave_barrier()
 using std::max;
 using std::min;
+
+namespace host_block {
+// Runs kern(params) for every workgroup of the grid in turn. A thread that returns from the kernel leaves the
+// barriers (as a finished wave does on the GPU), so kernels whose threads exit at different points still end.
+template <typename Kernel, typename Params>
+inline hipError_t launch(Kernel kern, dim3 grid, dim3 block, const Params& params, size_t lds_bytes) {
+  if (lds_bytes > kLdsBytes || block.x == 0 || block.x > 1024) return hipErrorUnknown;
+  blockDim = block;
+  gridDim = grid;
+  for (unsigned id = 0; id < grid.x; ++id) {
+    Block state(block.x);
+    current() = &state;
+    std::memset(dynamic_lds(), 0xFF, kLdsBytes);          // NaN patterns: nothing may be read before it is written
+    std::vector<std::thread> pool;
+    pool.reserve(block.x);
+    for (unsigned t = 0; t < block.x; ++t)
+      pool.emplace_back([&, t] {
+        threadIdx = dim3(t);
+        blockIdx = dim3(id);
+        kern(params);
+        state.all.arrive_and_drop();
+        state.wave[t / 64]->arrive_and_drop();
+      });
+    for (auto& th : pool) th.join();
+  }
+  current() = nullptr;
+  return hipSuccess;
+}
+}  // namespace host_block
+// `kern` and `Params` are the kernel pointer and the parameter type in the scope of the library's
+// launch_checked(), the only caller: the type-erased first argument cannot be called from here.
+#define hipLaunchKernel(fn, grid, block, args, lds_bytes, stream) host_block::launch(kern, grid, block, *static_cast<const Params*>((args)[0]), lds_bytes)
