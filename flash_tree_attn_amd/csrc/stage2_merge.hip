@@ -4,7 +4,8 @@
 //
 // One thread owns four consecutive head_dim columns of one output row; the row's
 // split weights exp(lse_s - max) are recomputed per thread (the split count is
-// small by construction of the heuristic), so no cross-lane traffic is needed.
+// small by construction of the heuristic). With many splits and few rows four
+// threads share the walk over the splits (see the kernel).
 #include "fta_device.h"
 
 namespace fta {
@@ -29,18 +30,27 @@ template <> struct Pack4<__bf16> {
   }
 };
 
-template <typename T, int D>
+// SG = 1: one thread owns four consecutive head_dim columns of one output row and walks all of the row's
+// splits. SG = 4: four threads share those columns and walk every fourth split each, their partial sums
+// meet in LDS. The second form is for calls with many splits and few rows (one long sequence): there the
+// first leaves the machine a few hundred waves that each issue their loads one split after the other.
+template <typename T, int D, int SG>
 __global__ void __launch_bounds__(256) stage2_merge_kernel(const KernelParams p) {
   constexpr int kThreadsPerRow = D / 4;
-  constexpr int kRowsPerBlock = 256 / kThreadsPerRow;
+  constexpr int kRowsPerBlock = 256 / (kThreadsPerRow * SG);
+  static_assert(kRowsPerBlock >= 1, "a row's threads fit one block");
   const int chunk = batch_chunk(p);   // the same cut stage 1 made (block-wide: before any thread leaves)
   const int64_t total_rows = static_cast<int64_t>(p.bsz) * p.num_q_heads * p.q_len;
-  const int64_t row = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + threadIdx.x / kThreadsPerRow;
-  if (row >= total_rows) return;
+  const int r_in_block = threadIdx.x / (kThreadsPerRow * SG);
+  const int g = (threadIdx.x / kThreadsPerRow) % SG;
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + r_in_block;
+  const bool valid = row < total_rows;
+  if (SG == 1 && !valid) return;
+  const int64_t row_c = valid ? row : 0;
   const int d = (threadIdx.x % kThreadsPerRow) * 4;
-  const int i = static_cast<int>(row % p.q_len);
-  const int head = static_cast<int>((row / p.q_len) % p.num_q_heads);
-  const int b = static_cast<int>(row / (static_cast<int64_t>(p.q_len) * p.num_q_heads));
+  const int i = static_cast<int>(row_c % p.q_len);
+  const int head = static_cast<int>((row_c / p.q_len) % p.num_q_heads);
+  const int b = static_cast<int>(row_c / (static_cast<int64_t>(p.q_len) * p.num_q_heads));
 
   const int S_b = splits_for(clamped_len(p, b), chunk, p.num_splits);
 
@@ -52,25 +62,47 @@ __global__ void __launch_bounds__(256) stage2_merge_kernel(const KernelParams p)
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   float wsum = 0.f;
   if (mx != neg_inf()) {
-    for (int s = 0; s < S_b; ++s) {
+    for (int s = g; s < S_b; s += SG) {
       const float wgt = fast_exp2((lse[s * p.mid_lse_stride[2]] - mx) * kLog2e);
       const f32x4 o = *reinterpret_cast<const f32x4*>(mo + s * p.mid_o_stride[2]);
       acc += wgt * o;
       wsum += wgt;
     }
-    acc *= 1.f / wsum;
   }
+  if constexpr (SG > 1) {
+    __shared__ f32x4 s_acc[kRowsPerBlock][SG][kThreadsPerRow];
+    __shared__ float s_w[kRowsPerBlock][SG];
+    s_acc[r_in_block][g][threadIdx.x % kThreadsPerRow] = acc;
+    if (threadIdx.x % kThreadsPerRow == 0) s_w[r_in_block][g] = wsum;
+    __syncthreads();
+    if (g != 0 || !valid) return;
+#pragma unroll
+    for (int o = 1; o < SG; ++o) {
+      acc += s_acc[r_in_block][o][threadIdx.x % kThreadsPerRow];
+      wsum += s_w[r_in_block][o];
+    }
+  }
+  if (mx != neg_inf()) acc *= 1.f / wsum;
   T* dst = static_cast<T*>(p.out) + b * p.out_stride[0] + head * p.out_stride[1] + i * p.out_stride[2] + d;
   Pack4<T>::store(dst, acc);
 }
 
-template <typename T, int D>
-int launch(const KernelParams& p, hipStream_t stream) {
-  constexpr int kRowsPerBlock = 256 / (D / 4);
+template <typename T, int D, int SG>
+int launch_sg(const KernelParams& p, hipStream_t stream) {
+  constexpr int kRowsPerBlock = 256 / ((D / 4) * SG);
   const int64_t total_rows = static_cast<int64_t>(p.bsz) * p.num_q_heads * p.q_len;
   const int64_t grid = (total_rows + kRowsPerBlock - 1) / kRowsPerBlock;
   if (grid <= 0 || grid > 0x7fffffffLL) return FTA_ERR_SHAPE;
-  return launch_checked(stage2_merge_kernel<T, D>, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, p);
+  return launch_checked(stage2_merge_kernel<T, D, SG>, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, p);
+}
+
+template <typename T, int D>
+int launch(const KernelParams& p, hipStream_t stream) {
+  // Waves the one-thread-per-column form would launch: below 16 per CU of a 256-CU part, with eight splits or
+  // more to walk, the walk is shared by four threads.
+  const int64_t waves = static_cast<int64_t>(p.bsz) * p.num_q_heads * p.q_len * (D / 4) / 64;
+  if (p.num_splits >= 8 && waves < 16 * kDefaultCUs) return launch_sg<T, D, 4>(p, stream);
+  return launch_sg<T, D, 1>(p, stream);
 }
 
 template <typename T>

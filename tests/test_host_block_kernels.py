@@ -168,6 +168,37 @@ def test_stage_entries_on_host_threads(host_lib):
     assert call.out[0, 0, 0].abs().max() == 0
 
 
+@pytest.mark.parametrize("dtype,D,L", [(torch.float32, 32, 3), (torch.bfloat16, 64, 5)])
+def test_stage2_with_the_walk_shared_by_four_threads(host_lib, dtype, D, L):
+    """Many splits, few rows (one long sequence): four threads share each row's walk over the splits and add
+    their partial sums in LDS. Rows that do not fill the last workgroup, dead splits, slots the sequence does
+    not reach, a row with no live split."""
+    bsz, hq, hkv, tmax, lens = 2, 2, 1, 2048, [2000, 700]
+    x = make(9, bsz, hq, hkv, L, D, tmax, dtype, lens)
+    call = HostCall(host_lib, x, splits=16)
+    S = call.plan.num_splits
+    assert S >= 8 and bsz * hq * L * (D // 4) // 64 < 16 * 256          # the launch takes the shared walk
+    chunk = call.plan.chunk_for(max(lens))
+    s_of = [live_splits(t, chunk, S) for t in lens]
+    assert s_of[0] == S and 1 < s_of[1] < S
+    whole = call.run().clone()                                          # stage 1 + stage 2 through it
+    torch.testing.assert_close(whole.float(), oracle(x), **TOL[dtype])
+    g = torch.Generator().manual_seed(6)
+    mid, lse = torch.randn(call.mid.shape, generator=g), torch.randn(call.lse.shape, generator=g) * 3
+    dead = torch.rand(lse.shape, generator=g) < 0.2
+    dead[1, 1, :, L - 1] = True
+    lse[dead], mid[dead] = -math.inf, 0.0
+    for b in range(bsz):
+        mid[b, :, s_of[b]:], lse[b, :, s_of[b]:] = float("nan"), float("nan")
+    call.mid.copy_(mid), call.lse.copy_(lse)
+    call.out.fill_(float("nan"))
+    call.run("fta_decode_stage2")
+    for b in range(bsz):
+        ref, _ = stage2_merge_oracle([mid[b, :, s].double() for s in range(s_of[b])], [lse[b, :, s].double() for s in range(s_of[b])])
+        torch.testing.assert_close(call.out[b].double(), ref, **TOL[dtype])
+    assert call.out[1, 1, L - 1].abs().max() == 0
+
+
 def test_paged_caches_and_packed_mask_on_host_threads(host_lib):
     lens, tmax, page = [150, 33], 192, 16
     x = make(7, 2, 4, 2, 6, 32, tmax, torch.float16, lens)
