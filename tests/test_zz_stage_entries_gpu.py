@@ -140,13 +140,15 @@ def test_stage1_alone_fills_the_slots_the_oracle_predicts(shape):
 
 # ---------------------------------------------------------------- stage 2 alone
 @pytest.mark.gpu
-@pytest.mark.parametrize("dtype,D", [(torch.float32, 64), (torch.bfloat16, 128), (torch.float16, 256), (torch.float32, 32)])
-def test_stage2_alone_merges_oracle_made_partials(dtype, D):
+@pytest.mark.parametrize("dtype,D,splits", [(torch.float32, 64, 6), (torch.bfloat16, 128, 6), (torch.float16, 256, 6), (torch.float32, 32, 6),
+                                            (torch.bfloat16, 128, 16), (torch.float32, 32, 16)])   # 16: the walk over the splits shared by four threads
+def test_stage2_alone_merges_oracle_made_partials(dtype, D, splits):
     bsz, hq, hkv, L, tmax = 4, 6, 3, 5, 2048
     lens = [2048, 700, 0, 1100]
     x = make(72, bsz, hq, hkv, L, D, tmax, dtype, lens)
-    pc = prepare(x, _force_splits=6)
+    pc = prepare(x, _force_splits=splits)
     S = pc.plan.num_splits
+    assert S == 6 if splits == 6 else S >= 8
     chunk = pc.plan.chunk_for(max(lens))
     s_of = [live_splits(t, chunk, S) for t in lens]
     assert S >= 4 and s_of[0] == S and 1 < s_of[1] < S and s_of[2] == 1      # full, partly filled and one-slot sequences
