@@ -204,8 +204,11 @@ int plan(const fta_args& a, int num_cus, fta_plan_out* out) {
   // Scratch the caller brought bounds what the heuristic may pick: a caller of the reference
   // sizes it from the batch's longest sequence (flash_tree_attn.py:274-281), which can be far
   // below the capacity this plan is cut for. (A forced count that does not fit stays an error.)
+  // Only where it binds: scratch sized from this plan's own answer leaves the plan as it is.
   const int64_t slots = a.mid_o && a.mid_lse && a.mid_splits > 0 ? a.mid_splits : 64;
-  const Cut cap_cut = cut_for(cap, std::min<int64_t>(64, slots), false);
+  const bool forced = a.force_splits > 0 || env_knobs().force_splits > 0;
+  Cut cap_cut = cut_for(cap, 64, false);
+  if (!forced && slots < cap_cut.splits) cap_cut = cut_for(cap, slots, false);
   const int64_t splits = cap_cut.splits, chunk = cap_cut.chunk;
   for (int i = 0; i < FTA_LEN_BUCKETS; ++i) {
     const int k = FTA_LEN_BUCKETS - 1 - i;   // steps below the cap

@@ -184,7 +184,11 @@ int fta_validate(const fta_args* args);
 /* The split-count heuristic that replaces "one split per block_size keys"
  * (flash_tree_attn.py:266-274, :293-299). Pure host code. `num_cus` is the number
  * of compute units to fill (256 on MI355X); pass 0 to use that default. Does not
- * look at kv_seq_len values (no host sync, unlike flash_tree_attn.py:272). */
+ * look at kv_seq_len values (no host sync, unlike flash_tree_attn.py:272). Scratch that is
+ * already in the arguments (mid_o, mid_lse, mid_splits) and holds fewer slots than the
+ * heuristic would take bounds its split count (a caller of the reference sizes it from the
+ * batch's longest sequence); scratch sized from this function's own answer changes nothing,
+ * so fta_decode, which plans from the arguments it is given, runs the plan reported here. */
 int fta_plan(const fta_args* args, int num_cus, fta_plan_out* plan);
 
 /* Runs the whole path (stage 1 with the tree block folded in, then the LSE merge

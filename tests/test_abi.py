@@ -359,3 +359,21 @@ def test_scratch_the_caller_brought_bounds_the_split_count(fta_lib):
     a.force_splits = 4                      # a pinned count is the caller's word: it is planned, and fta_decode refuses the scratch
     st, pl = plan(fta_lib, a)
     assert st == 0 and pl.num_splits == 4
+
+
+@pytest.mark.parametrize("kw", CASES)
+def test_plan_with_its_own_scratch_filled_in_is_stable(fta_lib, kw):
+    """A caller plans, allocates the slots the plan names, fills them in: the plan that fta_decode then makes from
+    those arguments is the same plan. Fewer slots bound it."""
+    a = base_args(**kw)
+    st, first = plan(fta_lib, a)
+    assert st == 0
+    a.mid_o = a.mid_lse = 0x1000
+    a.mid_splits = first.num_splits
+    st, second = plan(fta_lib, a)
+    assert st == 0 and bytes(second) == bytes(first)
+    a.mid_splits = max(1, first.num_splits - 1)              # one slot short: the plan shrinks to fit, and stays there
+    st, third = plan(fta_lib, a)
+    assert st == 0 and third.num_splits <= a.mid_splits
+    st, fourth = plan(fta_lib, a)
+    assert bytes(fourth) == bytes(third)
