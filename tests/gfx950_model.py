@@ -2,10 +2,16 @@
 (flash_tree_attn_amd/csrc/gen_wide_loop.py), so that the generated TEXT can be executed on the CPU:
 one workgroup of four 64-lane waves, their registers, one LDS array, a flat global memory, barriers.
 
-Test infrastructure only. It models results, not time: no latencies, no wait counters (every load
-completes at once; `s_waitcnt` and `s_nop` do nothing), so it finds wrong arithmetic, wrong
-registers, wrong addresses and wrong ring bookkeeping, and it cannot find a missing wait or an
-issue hazard (the generator's `verify()` / `hazards()` and the GPU tests are for those).
+Test infrastructure only. It models results, not time: every load delivers its data at once. What it
+does keep is the BOOKKEEPING of the wait counters, so that a missing wait is an error even though the
+data would have been there:
+  * LDS reads retire in order; a register that a read has not delivered yet (no `s_waitcnt lgkmcnt(n)`
+    has covered it) may not be named by any other instruction;
+  * tile requests (global_load_lds) retire in order per wave; the LDS bytes of a request are readable by
+    the requesting wave once its `s_waitcnt vmcnt(n)` has covered the request, and by the other waves
+    after the next barrier behind that wait; a read of bytes that are still in flight, or a request into
+    bytes that any wave reads between the same two barriers, is an error (the ring's stages are reused).
+Issue hazards (wait states between dependent instructions) are the generator's `hazards()` check.
 
 Lane layouts of the matrix instruction v_mfma_f32_32x32x16_{bf16,f16} (D = A.B + C, A 32x16, B 16x32):
 lane l holds, of A, row l % 32 and the 8 values k = 8 * (l // 32) .. + 7 (four registers, two values
@@ -73,6 +79,12 @@ class Wave:
         self.lds, self.mem, self.dtype = lds, mem, dtype
         self.executed = 0
         self.taken = []          # labels branched to (in order), for tests that want to see a path taken
+        self.lds_pending = []    # destination registers of LDS reads no lgkmcnt wait has covered yet, oldest first
+        self.vm_pending = []     # (lo, hi) LDS byte ranges of tile requests no vmcnt wait has covered yet, oldest first
+        self.vm_own = []         # ranges whose wait this wave has passed, not yet published to the others by a barrier
+        self.epoch_reads = []    # (lo, hi) LDS ranges read since the last barrier
+        self.epoch_requests = [] # (lo, hi) LDS ranges requested into since the last barrier, with the reads that preceded them
+        self.shared = None       # the workgroup's bookkeeping (set by run_workgroup)
 
     # ---- operands
     def _reg(self, tok):
@@ -159,6 +171,26 @@ class Wave:
             D = (A.astype(np.float64) @ B.astype(np.float64) + C.astype(np.float64)).astype(np.float32)
         fd[ld:ld + 16] = D[rows, cols].view(np.uint32)
 
+    # ---- bookkeeping of the wait counters (see the module text)
+    def note_lds_read(self, addr, nbytes, text):
+        lo, hi = int(addr.min()), int(addr.max()) + nbytes
+        for other in (self.shared or [self]):
+            busy = other.vm_pending + ([] if other is self else other.vm_own)
+            for r_lo, r_hi in busy:
+                if lo < r_hi and hi > r_lo and bool(((addr < r_hi) & (addr + nbytes > r_lo)).any()):
+                    who = "this wave has not waited for" if other is self else "another wave has not published"
+                    raise RuntimeError(f"`{text}` reads LDS bytes {r_lo}..{r_hi} of a tile request that {who}")
+        self.epoch_reads.append((lo, hi))
+
+    def note_request(self, lo, hi, text):
+        for other in (self.shared or []):
+            if other is self:
+                continue
+            for r_lo, r_hi in other.epoch_reads:
+                if lo < r_hi and hi > r_lo:
+                    raise RuntimeError(f"`{text}` requests a tile into LDS bytes {lo}..{hi} that another wave reads before the next barrier")
+        self.vm_pending.append((lo, hi))
+
     # ---- LDS
     def lds_read(self, addr, nbytes):
         out = np.zeros((LANES, nbytes), dtype=np.uint8)
@@ -168,6 +200,19 @@ class Wave:
                 raise IndexError(f"LDS read at {a} outside the array")
             out[l] = self.lds[a:a + nbytes]
         return out
+
+
+_VREG_RE = re.compile(r"\b([va])(\d+)\b|\b([va])\[(\d+):(\d+)\]")
+
+
+def _vector_regs(text):
+    out = set()
+    for m in _VREG_RE.finditer(text.split(";")[0]):
+        if m.group(1):
+            out.add((m.group(1), int(m.group(2))))
+        else:
+            out.update((m.group(3), i) for i in range(int(m.group(4)), int(m.group(5)) + 1))
+    return frozenset(out)
 
 
 def _strip(op):
@@ -188,13 +233,31 @@ def run_wave(w: Wave, body):
         ins.append((_strip(parts[0]), [x.strip() for x in parts[1].split(",")] if len(parts) > 1 else [], line))
     pc = 0
     fmax = lambda x, y: np.fmax(x, y)
+    named = [_vector_regs(text) if op[0] in "vdg" else frozenset() for op, _, text in ins]   # vector registers each instruction names
     with np.errstate(all="ignore"):
         while pc < len(ins):
             op, a, text = ins[pc]
+            touched = named[pc]
             pc += 1
             w.executed += 1
-            if op in ("s_nop", "s_waitcnt"):
+            if op == "s_nop":
                 continue
+            if op == "s_waitcnt":
+                m = re.search(r"lgkmcnt\((\d+)\)", text)
+                if m:
+                    w.lds_pending = w.lds_pending[len(w.lds_pending) - int(m.group(1)):] if int(m.group(1)) else []
+                m = re.search(r"vmcnt\((\d+)\)", text)
+                if m:
+                    keep = int(m.group(1))
+                    done = len(w.vm_pending) - keep
+                    if done > 0:
+                        w.vm_own += w.vm_pending[:done]
+                        w.vm_pending = w.vm_pending[done:]
+                continue
+            if w.lds_pending and touched:
+                for dest in w.lds_pending:
+                    if dest & touched:
+                        raise RuntimeError(f"`{text}` names a register of an LDS read that no lgkmcnt wait has covered")
             if op == "s_barrier":
                 yield "barrier"
             elif op == "s_branch":
@@ -306,6 +369,8 @@ def run_wave(w: Wave, body):
                 addr_tok, off = a[1].split() if " " in a[1] else (a[1], "offset:0")
                 addr = w.src32(addr_tok).astype(np.int64) + int(off.split(":")[1], 0)
                 fd, ld, nd = w.tuple_regs(a[0])
+                w.note_lds_read(addr, 16 if op == "ds_read_b128" else 8, text)
+                w.lds_pending.append(frozenset(("v" if fd is w.v else "a", ld + i) for i in range(nd)))
                 if op == "ds_read_b128":
                     assert nd == 4
                     fd[ld:ld + 4] = w.lds_read(addr, 16).view(np.uint32).reshape(LANES, 4).T
@@ -321,6 +386,7 @@ def run_wave(w: Wave, body):
                 lo = w._reg(a[1])[2]
                 base = int(w.s[lo]) | (int(w.s[lo + 1]) << 32)
                 off = w.src32(a[0])
+                w.note_request(w.m0, w.m0 + 16 * LANES, text)
                 for l in range(LANES):
                     dst = w.m0 + 16 * l
                     if dst + 16 > w.lds.size:
@@ -334,6 +400,9 @@ def run_workgroup(waves, bodies):
     """Runs the waves of one workgroup to completion; all live waves meet at every barrier. `bodies[i]` is
     the instruction text of wave i (waves may run different statements with the same barrier count)."""
     gens = [run_wave(w, b) for w, b in zip(waves, bodies)]
+    for w in waves:
+        w.shared = waves
+        w.epoch_reads = []
     live = list(range(len(gens)))
     barriers = 0
     while live:
@@ -348,4 +417,7 @@ def run_workgroup(waves, bodies):
             raise RuntimeError(f"waves {done} finished while waves {arrived} wait at a barrier")
         barriers += bool(arrived)
         live = arrived
+        for w in waves:       # behind the barrier: what each wave had waited for is everybody's, and a new span of reads begins
+            w.vm_own = []
+            w.epoch_reads = []
     return barriers

@@ -348,3 +348,55 @@ def test_a_whole_split_tree_tiles_loop_and_ragged_tail(D, dtype, L, heads, full_
     np.testing.assert_allclose(((m + np.log2(l)) * math.log(2.0))[:rows], ref_lse, atol=2e-3, rtol=0)
     np.testing.assert_allclose((o / l[:, None])[:rows], ref, atol=2e-3, rtol=1e-2)
     assert np.isfinite(o).all() and np.isfinite(l).all()    # rows past the unit (zero queries) stay finite too
+
+
+def _run_mutated(mutate, D=64, dtype="bf16", tiles=8):
+    q, k, v = make_case(1, D, tiles)
+    wg = Workgroup(D, dtype, q, k, v)
+    wg.setup(tiles, 1.0 / math.sqrt(D))
+    body = mutate(list(GEN.gen(D, dtype)))
+    run_workgroup(wg.waves, [body] * NW)
+
+
+def test_the_model_holds_the_loop_to_its_waits():
+    """The model delivers every load at once, but keeps the books of the wait counters: a text whose waits are
+    weaker than its reads need, or whose requests overtake the barrier, must fail although the data is there."""
+    import re
+    _run_mutated(lambda b: b)                                            # as rendered: clean
+    base = GEN.gen(64, "bf16")
+    stop = next(i for i, l in enumerate(base) if l.startswith(".Lfix0"))
+    waits = [i for i, l in enumerate(base) if l.startswith("s_waitcnt lgkmcnt") and i < stop]
+    assert len(waits) >= 20
+    for i in waits[::3]:                                                 # every wait is exactly as strong as it must be
+        def weaker(b, i=i):
+            n = int(re.search(r"\((\d+)\)", b[i]).group(1))
+            b[i] = f"s_waitcnt lgkmcnt({n + 1})"
+            return b
+        with pytest.raises(RuntimeError, match="no lgkmcnt wait has covered"):
+            _run_mutated(weaker, tiles=2)
+
+    def weaker_tile_wait(b):
+        i = next(i for i, l in enumerate(b) if l.startswith("s_waitcnt vmcnt"))
+        n = int(re.search(r"\((\d+)\)", b[i]).group(1))
+        b[i] = f"s_waitcnt vmcnt({n * 3 // 2})"                          # leaves three tiles in flight instead of two
+        return b
+    with pytest.raises(RuntimeError, match="this wave has not waited for"):
+        _run_mutated(weaker_tile_wait)
+
+    def no_barrier(b):
+        b[b.index("s_barrier")] = "s_nop 0"
+        return b
+    with pytest.raises(RuntimeError, match="another wave has not published"):
+        _run_mutated(no_barrier)
+
+    def request_ahead_of_the_barrier(b):
+        bar = b.index("s_barrier")
+        load = next(i for i, l in enumerate(b) if l.startswith("global_load_lds"))
+        group = b[load - 3:load + 1]                                     # address, M0, gap, request
+        del b[load - 3:load + 1]
+        where = next(i for i, l in enumerate(b) if l.startswith(f"s_add_u32 s{GEN.S_TMP + 6}"))
+        landing = b.pop(where)                                           # the LDS address the request lands at
+        b[bar:bar] = [landing] + group
+        return b
+    with pytest.raises(RuntimeError):
+        _run_mutated(request_ahead_of_the_barrier)
