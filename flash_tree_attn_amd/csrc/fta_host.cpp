@@ -186,7 +186,9 @@ int plan(const fta_args& a, int num_cus, fta_plan_out* out) {
     // latency-bound step worth about three cache tiles per tree tile): count it as extra
     // keys when cutting chunks, so that the last split of a full-length sequence gets a
     // correspondingly shorter cache range.
-    const int64_t tree_weight = env_knobs().tree_tile_weight >= 0 ? env_knobs().tree_tile_weight : 3;
+    // The 64-row-wave loop runs its cache tiles faster (1.9-2.1 us against 2.36) and its tree tiles slower
+    // (unpipelined masked halves, 13-16 us per tree tile in the kernel's own clock reads): 7 tiles' worth.
+    const int64_t tree_weight = env_knobs().tree_tile_weight >= 0 ? env_knobs().tree_tile_weight : wide ? 7 : 3;
     const int64_t tree_keys = splits > 1 ? tree_weight * kKeyTile * cdiv(a.q_len, kKeyTile) : 0;
     int64_t chunk = cdiv(cdiv(t_len + tree_keys, splits), gran) * gran;
     if ((splits - 1) * chunk >= t_len) chunk = cdiv(cdiv(t_len, splits), gran) * gran;
