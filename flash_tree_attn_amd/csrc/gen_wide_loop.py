@@ -419,6 +419,8 @@ def gen_masked(D: int, dtype: str, H: int) -> list[str]:
         e(f"v_cmp_neq_f32_e32 vcc, 0xff800000, {vr(t + 2)}")
         e(f"v_cndmask_b32_e32 {vr(t + 3)}, 0, {vr(t + 2)}, vcc")                # m_use: 0 while everything is masked
         al = V_E + 6 + qb                                                       # alpha of this row block (kept for O)
+        e(f"v_cmp_neq_f32_e32 vcc, 0xff800000, {vr(V_M + qb)}")                 # rows that have seen a key before: only their O needs rescaling
+        e(f"s_mov_b64 s[{S_TMP + 2 * qb}:{S_TMP + 2 * qb + 1}], vcc")
         e(f"v_sub_f32 {vr(al)}, {vr(V_M + qb)}, {vr(t + 3)}")
         e(f"v_exp_f32_e32 {vr(al)}, {vr(al)}")
         e(f"v_mov_b32 {vr(V_M + qb)}, {vr(t + 2)}")
@@ -447,10 +449,12 @@ def gen_masked(D: int, dtype: str, H: int) -> list[str]:
             e(f"v_sub_f32 {vr(e1)}, {vr(e1)}, {vr(f1)}")
             e(f"{cvt} {vr(rw)}, {vr(e0)}, {vr(e1)}")
         e(f"v_add_f32 {vr(V_L + qb)}, {vr(V_L + qb)}, {vr(t + 4)}")
-    # ---- rescale O where some row's reference moved
+    # ---- rescale O where the reference of a row that already holds something moved (a row without keys so far holds
+    # zeros whatever its alpha: the first half of a tree block skips the whole pass)
     e(f"v_cmp_neq_f32_e32 vcc, 1.0, {vr(V_E + 6)}")
-    e(f"s_mov_b64 s[{S_TMP + 4}:{S_TMP + 5}], vcc")
+    e(f"s_and_b64 s[{S_TMP + 4}:{S_TMP + 5}], vcc, s[{S_TMP}:{S_TMP + 1}]")
     e(f"v_cmp_neq_f32_e32 vcc, 1.0, {vr(V_E + 7)}")
+    e(f"s_and_b64 vcc, vcc, s[{S_TMP + 2}:{S_TMP + 3}]")
     e(f"s_or_b64 vcc, vcc, s[{S_TMP + 4}:{S_TMP + 5}]")
     e("s_cbranch_vccz .Lnoscale_%=")
     for qb in range(2):

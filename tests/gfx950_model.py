@@ -281,12 +281,19 @@ def run_wave(w: Wave, body):
                 else:
                     d, s_ = w._reg(a[0])[2], w._reg(a[1])[2]
                     w.s[d], w.s[d + 1] = w.s[s_], w.s[s_ + 1]
-            elif op == "s_or_b64":
-                assert a[0] == "vcc" and a[1] == "vcc"
-                lo = w._reg(a[2])[2]
-                bits = int(w.s[lo]) | (int(w.s[lo + 1]) << 32)
-                w.vcc = w.vcc | np.array([(bits >> i) & 1 == 1 for i in range(LANES)])
-                w.scc = int(w.vcc.any())
+            elif op in ("s_or_b64", "s_and_b64"):
+                def mask64(tok):
+                    if tok == "vcc":
+                        return sum(1 << i for i in range(LANES) if w.vcc[i])
+                    lo = w._reg(tok)[2]
+                    return int(w.s[lo]) | (int(w.s[lo + 1]) << 32)
+                bits = mask64(a[1]) | mask64(a[2]) if op == "s_or_b64" else mask64(a[1]) & mask64(a[2])
+                if a[0] == "vcc":
+                    w.vcc = np.array([(bits >> i) & 1 == 1 for i in range(LANES)])
+                else:
+                    lo = w._reg(a[0])[2]
+                    w.s[lo], w.s[lo + 1] = bits & 0xFFFFFFFF, bits >> 32
+                w.scc = int(bits != 0)
             elif op == "s_add_u32":
                 r = w.scalar(a[1]) + w.scalar(a[2])
                 w.scc = int(r > 0xFFFFFFFF)

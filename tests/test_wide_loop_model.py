@@ -324,8 +324,10 @@ def test_a_whole_split_tree_tiles_loop_and_ragged_tail(D, dtype, L, heads, full_
     wg.fill_edge_stage(0, 0, tk_store, 0, L)
     wg.fill_edge_stage(wg.kvring, 0, tv_store, 0, L)
     wg.run_masked_half(0, 0, 0, L, add)
+    assert all(w.taken == [".Lnoscale_%="] for w in wg.waves)         # nothing accumulated yet: O is not rescaled
     if 32 < L:
         wg.run_masked_half(1, 0, 32, L, add)
+        assert any(len(w.taken) == 1 for w in wg.waves)               # some row's reference moved: this time it is
     # phase B
     if full_tiles:
         wg.setup_loop(full_tiles)
