@@ -1,0 +1,40 @@
+"""The host build of the library's non-matrix kernels and host side (tests/host_block/) under the address,
+undefined-behaviour and thread sanitizers (GPU sanitizers do not exist on the target; host code is where
+they run). tests/host_block/sanitize_main.cpp calls fta_plan / fta_decode on buffers of exactly their size
+(contiguous and paged caches, ragged tiles, empty and over-long sequences, additive and packed masks) and
+checks the results against a plain double-precision attention.
+  * address / undefined: a read or write one element past a tensor, a page, the scratch, an LDS array;
+  * thread: every GPU thread is a host thread here and the only synchronisation is what the kernels ask for
+    (`__syncthreads`, wave barriers, shuffles), so a missing barrier is a data race the sanitizer reports
+    (checked by hand: without the barrier in front of the ranking loop of item_by_order it reports 12)."""
+import os
+import subprocess
+
+import pytest
+
+from flash_tree_attn_amd import build as fta_build
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CLANG = os.path.join(os.path.dirname(fta_build.HIPCC), "..", "llvm", "bin", "clang++")
+SOURCES = ["fta_host.cpp", "stage1_shuffle.hip", "stage2_merge.hip", "append_kv.hip"]
+
+
+@pytest.mark.parametrize("sanitize", ["address,undefined", "thread"])
+def test_host_build_is_clean_under(sanitize, tmp_path):
+    if not os.path.exists(CLANG):
+        pytest.skip("no host clang++")
+    flags = ["-x", "c++", "-std=c++20", "-O1", "-g", f"-fsanitize={sanitize}", "-fno-omit-frame-pointer", "-pthread",
+             "-I", os.path.join(HERE, "host_block"), "-I", fta_build.INCLUDE, "-I", fta_build.CSRC]
+    objs = []
+    for src in [os.path.join(fta_build.CSRC, s) for s in SOURCES] + [os.path.join(HERE, "host_block", n) for n in ("mfma_stub.cpp", "sanitize_main.cpp")]:
+        obj = str(tmp_path / (os.path.basename(src) + ".o"))
+        subprocess.run([CLANG, *flags, "-c", src, "-o", obj], check=True, capture_output=True)
+        objs.append(obj)
+    exe = str(tmp_path / "sanitize_host")
+    subprocess.run([CLANG, f"-fsanitize={sanitize}", "-pthread", *objs, "-o", exe], check=True, capture_output=True)
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0", UBSAN_OPTIONS="halt_on_error=1", TSAN_OPTIONS="halt_on_error=0")
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=900, env=env)
+    text = r.stdout + r.stderr
+    for sign in ("AddressSanitizer", "runtime error", "data race", "ThreadSanitizer", "FAILED"):
+        assert sign not in text, text[-3000:]
+    assert r.returncode == 0 and text.strip().endswith("clean"), text[-2000:]
