@@ -162,6 +162,7 @@ int main() {
       {1, 2, 2, 7, 32, 64, 1, 0, {64}, false},                // exactly one tile, one split
       {2, 4, 2, 4, 32, 90, 2, 16, {90, 17}, false},           // paged, the last page partly used
       {3, 2, 2, 2, 32, 48, 0, 16, {48, 1, 500}, true},        // paged, a length beyond the capacity, heuristic split count
+      {2, 2, 1, 3, 32, 1100, 16, 0, {1100, 300}, false},      // nine splits: stage 2 shares each row's walk between four threads
   };
   int bad = 0;
   for (const Case& c : cases) bad += run(c);
