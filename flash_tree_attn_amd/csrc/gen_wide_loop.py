@@ -685,7 +685,8 @@ def hazards(body: list[str], name: str) -> None:
 
 
 def render() -> str:
-    lines = ["// Generated by gen_wide_loop.py - do not edit; edit the generator and run it.", "// clang-format off"]
+    lines = ["// Generated by gen_wide_loop.py - do not edit; edit the generator and run it.", "// clang-format off",
+             "#ifndef FTA_WIDE_LOOP_ASM_INC", "#define FTA_WIDE_LOOP_ASM_INC"]
     for D in (128, 64):
         L = layout(D)
         for dtype in ("bf16", "f16"):
@@ -707,6 +708,7 @@ def render() -> str:
         lines.append(f"static_assert(fta::TileLayout<{D}>::kTileBytes == {L['tile']} && fta::TileLayout<{D}>::kBlockPitch == {L['pitch']} && "
                      f"fta::TileLayout<{D}>::kChunkStride == {L['chunk']} && fta::TileLayout<{D}>::kRowsPerBlock == {L['rpb']}, "
                      f"\"gen_wide_loop.py and TileLayout<{D}> disagree\");")
+    lines.append("#endif  // FTA_WIDE_LOOP_ASM_INC")
     lines.append("// clang-format on")
     return "\n".join(lines) + "\n"
 

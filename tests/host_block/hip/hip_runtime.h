@@ -51,6 +51,7 @@ struct Block {
 };
 inline Block*& current() { static Block* b = nullptr; return b; }
 inline char* dynamic_lds() { alignas(16) static char lds[kLdsBytes]; return lds; }
+inline size_t& lds_limit() { static size_t bytes = 0; return bytes; }   // dynamic LDS the running launch asked for
 }  // namespace host_block
 #define FTA_DYNAMIC_LDS(name) char* name = host_block::dynamic_lds()
 
@@ -99,6 +100,7 @@ inline hipError_t launch(Kernel kern, dim3 grid, dim3 block, const Params& param
   if (lds_bytes > kLdsBytes || block.x == 0 || block.x > 1024) return hipErrorUnknown;
   blockDim = block;
   gridDim = grid;
+  lds_limit() = lds_bytes;
   for (unsigned id = 0; id < grid.x; ++id) {
     Block state(block.x);
     current() = &state;

@@ -16,10 +16,32 @@ struct Case {
   int bsz, hq, hkv, L, D, tmax, splits, page;   // page 0 = contiguous caches
   std::vector<long long> lens;
   bool packed;
+  bool mfma = false;    // bf16 tensors through the MFMA kernel (where the build has it) instead of fp32 through the shuffle kernel
+  bool fused = false;   // with counters: the merge inside stage 1's launch
 };
 
 std::mt19937 rng(1234);
 float rnd() { return std::normal_distribution<float>(0.f, 1.f)(rng); }
+uint16_t to_bf16(float x) {
+  uint32_t u;
+  std::memcpy(&u, &x, 4);
+  return static_cast<uint16_t>((u + 0x7FFF + ((u >> 16) & 1)) >> 16);
+}
+float from_bf16(uint16_t h) {
+  const uint32_t u = static_cast<uint32_t>(h) << 16;
+  float x;
+  std::memcpy(&x, &u, 4);
+  return x;
+}
+// Rounds `t` to bf16 in place (the reference then sees what the library sees) and returns the 16-bit tensor; NaN stays NaN.
+std::vector<uint16_t> as_bf16(std::vector<float>& t) {
+  std::vector<uint16_t> h(t.size());
+  for (size_t i = 0; i < t.size(); ++i) {
+    h[i] = std::isnan(t[i]) ? uint16_t{0x7FC0} : to_bf16(t[i]);
+    t[i] = from_bf16(h[i]);
+  }
+  return h;
+}
 
 int run(const Case& c) {
   const int G = c.hq / c.hkv;
@@ -61,14 +83,30 @@ int run(const Case& c) {
       }
   }
 
+  std::vector<uint16_t> q16, ck16, cv16, k16, v16, kp16, vp16, out16;
+  if (c.mfma) {
+    q16 = as_bf16(q); ck16 = as_bf16(ck); cv16 = as_bf16(cv);
+    if (c.page) { kp16 = as_bf16(kp); vp16 = as_bf16(vp); }
+    k16 = as_bf16(k); v16 = as_bf16(v);       // rounded also when paged: the reference reads k and v
+    if (c.page) { k16.clear(); v16.clear(); k16.shrink_to_fit(); v16.shrink_to_fit(); }
+    out16.assign(out.size(), 0x7FC0);
+  }
   fta_args a{};
-  a.q = q.data(); a.cur_k = ck.data(); a.cur_v = cv.data(); a.kv_seq_len = c.lens.data(); a.out = out.data();
-  a.k_cache = c.page ? kp.data() : k.data();
-  a.v_cache = c.page ? vp.data() : v.data();
+  a.kv_seq_len = c.lens.data();
+  if (c.mfma) {
+    a.q = q16.data(); a.cur_k = ck16.data(); a.cur_v = cv16.data(); a.out = out16.data();
+    a.k_cache = c.page ? kp16.data() : k16.data();
+    a.v_cache = c.page ? vp16.data() : v16.data();
+  } else {
+    a.q = q.data(); a.cur_k = ck.data(); a.cur_v = cv.data(); a.out = out.data();
+    a.k_cache = c.page ? kp.data() : k.data();
+    a.v_cache = c.page ? vp.data() : v.data();
+  }
   a.mask = c.packed ? (const void*)bits.data() : (const void*)mask.data();
   a.mask_kind = c.packed ? FTA_MASK_PACKED_U64 : FTA_MASK_ADDITIVE_F32;
   a.bsz = c.bsz; a.num_q_heads = c.hq; a.num_kv_heads = c.hkv; a.cur_heads = c.hkv; a.q_len = c.L; a.head_dim = c.D;
-  a.block_size = 64; a.dtype = FTA_F32; a.len_dtype = FTA_I64; a.force_splits = c.splits; a.force_kernel = FTA_KERNEL_SHUFFLE;
+  a.block_size = 64; a.dtype = c.mfma ? FTA_BF16 : FTA_F32; a.len_dtype = FTA_I64; a.force_splits = c.splits;
+  a.force_kernel = c.mfma ? FTA_KERNEL_MFMA : FTA_KERNEL_SHUFFLE;
   a.sm_scale = 1.f / std::sqrt((float)c.D);
   const long long LD = (long long)c.L * c.D;
   a.q_stride[0] = c.hq * LD; a.q_stride[1] = LD; a.q_stride[2] = c.D;
@@ -92,7 +130,14 @@ int run(const Case& c) {
     a.mid_o_stride[0] = (long long)c.hq * pl.num_splits * LD; a.mid_o_stride[1] = pl.num_splits * LD; a.mid_o_stride[2] = LD; a.mid_o_stride[3] = c.D;
     a.mid_lse_stride[0] = (long long)c.hq * pl.num_splits * c.L; a.mid_lse_stride[1] = (long long)pl.num_splits * c.L; a.mid_lse_stride[2] = c.L;
   }
+  std::vector<int32_t> counters(c.fused ? (size_t)pl.counter_elems : 0, 0);
+  if (c.fused) {
+    if (pl.counter_elems <= 0) { std::printf("no merge inside the launch for this case\n"); return 1; }
+    a.counters = counters.data(); a.counter_elems = pl.counter_elems;
+  }
   if (int st = fta_decode(&a, nullptr)) { std::printf("decode failed %d\n", st); return 1; }
+  for (int32_t n : counters) if (n != 0) { std::printf("a counter was left at %d\n", n); return 1; }
+  if (c.mfma) for (size_t i = 0; i < out.size(); ++i) out[i] = from_bf16(out16[i]);
 
   // plain attention in double
   double worst = 0;
@@ -118,13 +163,17 @@ int run(const Case& c) {
           const float* vr = j < T ? &v[(((size_t)b * c.hkv + h / G) * c.tmax + j) * c.D] : &cv[(((size_t)b * c.hkv + h / G) * c.L + (j - T)) * c.D];
           for (int e = 0; e < c.D; ++e) o[e] += p * vr[e];
         }
-        for (int e = 0; e < c.D; ++e)
-          worst = std::max(worst, std::fabs(o[e] / den - out[(((size_t)b * c.hq + h) * c.L + i) * c.D + e]));
+        for (int e = 0; e < c.D; ++e) {
+          const double ref = o[e] / den, got = out[(((size_t)b * c.hq + h) * c.L + i) * c.D + e];
+          const double err = std::fabs(ref - got);                      // NaN (an element never written) must fail
+          worst = err == err ? std::max(worst, c.mfma ? err / (1.0 + 5.0 * std::fabs(ref)) : err) : INFINITY;
+        }
       }
   }
-  std::printf("bsz %d hq %d hkv %d L %d D %d tmax %d splits %d page %d packed %d: plan %d x %d, max abs err %.2e\n", c.bsz, c.hq, c.hkv, c.L, c.D,
-              c.tmax, c.splits, c.page, (int)c.packed, pl.num_splits, pl.chunk, worst);
-  return worst < 2e-5 ? 0 : 1;
+  std::printf("%s bsz %d hq %d hkv %d L %d D %d tmax %d splits %d page %d packed %d: plan %d x %d, %d rows per workgroup, max abs err %.2e\n",
+              c.mfma ? "bf16/mfma" : "fp32/shuffle", c.bsz, c.hq, c.hkv, c.L, c.D, c.tmax, c.splits, c.page, (int)c.packed, pl.num_splits, pl.chunk,
+              pl.rows_per_wg, worst);
+  return worst < (c.mfma ? 2e-3 : 2e-5) ? 0 : 1;   // bf16: 2e-3 absolute + 1e-2 relative, as everywhere
 }
 // The accepted-path append on exactly sized caches, one sequence running into the end of its cache.
 int run_append() {
@@ -155,7 +204,16 @@ int run_append() {
 }
 }  // namespace
 
-int main() {
+int main(int argc, char** argv) {
+  // "mfma" as first argument: the build holds the MFMA kernel (stage1_mfma_host.cpp), run its cases as well
+  const bool with_mfma = argc > 1 && std::strcmp(argv[1], "mfma") == 0;
+  const Case mfma_cases[] = {
+      {2, 4, 2, 5, 64, 200, 2, 0, {200, 77}, false, true},                 // 4 waves, rings of 2; ragged last tiles
+      {1, 8, 1, 20, 128, 390, 1, 0, {390}, false, true},                   // 8 waves pipelined through rings of 3 and 5, ragged end
+      {2, 2, 2, 3, 128, 160, 2, 16, {160, 17}, true, true},                // paged, packed mask
+      {2, 8, 1, 20, 64, 192, 3, 0, {192, 70}, false, true, true},          // pipelined, merge inside the launch
+      {1, 2, 2, 3, 256, 65, 1, 0, {65}, false, true},                      // head_dim 256, one key past a tile
+  };
   const Case cases[] = {
       {2, 4, 2, 5, 32, 100, 2, 0, {100, 37}, false},          // ragged tiles at the end of cache and tree
       {2, 2, 1, 3, 64, 129, 3, 0, {129, 0}, true},            // one key past a tile boundary; an empty cache; packed mask
@@ -166,6 +224,8 @@ int main() {
   };
   int bad = 0;
   for (const Case& c : cases) bad += run(c);
+  if (with_mfma)
+    for (const Case& c : mfma_cases) bad += run(c);
   bad += run_append();
   std::printf(bad ? "FAILED\n" : "clean\n");
   return bad;

@@ -67,7 +67,7 @@ def make(seed, bsz, hq, hkv, L, D, tmax, dtype, lens):
 class HostCall:
     """fta_args over CPU tensors (what flash_decoding.prepare does for device tensors), planned, with scratch."""
 
-    def __init__(self, lib, x, splits=0, hint=0, mask=None, tables=None, pools=None):
+    def __init__(self, lib, x, splits=0, hint=0, mask=None, tables=None, pools=None, kernel=_lib.KERNEL_SHUFFLE, counters=False):
         self.lib, self.x = lib, x
         q = x["q"]
         bsz, hq, L, D = q.shape
@@ -86,7 +86,7 @@ class HostCall:
         else:
             a.cache_len = a.v_cache_len = k.size(2)
         a.block_size, a.max_seq_len_hint, a.dtype, a.len_dtype = 64, hint, DTYPES[q.dtype], _lib.FTA_I64
-        a.force_splits, a.force_kernel, a.sm_scale = splits, _lib.KERNEL_SHUFFLE, 1.0 / math.sqrt(D)
+        a.force_splits, a.force_kernel, a.sm_scale = splits, kernel, 1.0 / math.sqrt(D)
         for name, t in (("q_stride", q), ("k_stride", k), ("v_stride", v), ("ck_stride", x["current_k"]), ("cv_stride", x["current_v"]), ("out_stride", self.out)):
             getattr(a, name)[:] = t.stride()[:3]
         if mask.dtype == torch.int64:
@@ -102,6 +102,9 @@ class HostCall:
         a.mid_o, a.mid_lse, a.mid_splits = self.mid.data_ptr(), self.lse.data_ptr(), S
         a.mid_o_stride[:] = self.mid.stride()[:4]
         a.mid_lse_stride[:] = self.lse.stride()[:3]
+        if counters:      # zeroed once by the caller, left at zero by every call: stage 1 then merges in its own launch
+            self.counters = torch.zeros(bsz * hq * 4, dtype=torch.int32)
+            a.counters, a.counter_elems = self.counters.data_ptr(), self.counters.numel()
         self.args = a
 
     def run(self, entry="fta_decode"):

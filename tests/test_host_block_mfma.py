@@ -1,0 +1,180 @@
+"""The MFMA stage-1 kernel's SOURCE on host threads, against the oracle.
+
+tests/host_block/stage1_mfma_host.cpp compiles flash_tree_attn_amd/csrc/stage1_mfma.hip for the host with
+the instruction wrappers of csrc/gfx950_ops.h replaced by arithmetic stand-ins (gfx950_ops_host.h: the
+32x32x16 matrix product in its lane layout, the transposing LDS read, the direct global->LDS load with
+bounds-checked LDS addresses, ...), one host thread per GPU thread, and runs it through the library's own C
+entry points. All three compiled loop variants run: 4 waves x 32 rows with rings of 2 (also head_dim 256),
+and 8 waves x 32 rows software-pipelined over whole tiles. The assembly loop of 64-row waves does not exist
+on the host (tests/test_wide_loop_model.py executes that one).
+
+What this pins without a GPU: the work decomposition and addressing of the kernel (units, row blocks, splits,
+chunk by the batch's longest sequence, strides, paged lookups, ragged and tree tiles, the ring slots), its
+lane layouts, the online softmax with the deferred rescale, the compensated masked tiles, the epilogue, and
+the merge inside the launch with counters. What it cannot show: anything about time (loads land at once here,
+so wait counts are not exercised), and the last bits of the hardware's accumulation order.
+
+TEST INFRASTRUCTURE ONLY: nothing under flash_tree_attn_amd/ knows of this build."""
+import ctypes as C
+import math
+import os
+import subprocess
+
+import pytest
+import torch
+
+from flash_tree_attn_amd import _lib
+from flash_tree_attn_amd import build as fta_build
+from flash_tree_attn_amd.tree_mask import pack_mask
+from oracle.tree_attn_oracle import tree_attention_oracle
+from test_host_block_kernels import CLANG, HERE, SOURCES, TOL, HostCall, make, oracle
+from test_zz_stage_entries_gpu import expected_partials, live_splits
+
+MFMA = _lib.KERNEL_MFMA
+
+
+@pytest.fixture(scope="module")
+def host_lib(tmp_path_factory):
+    if not os.path.exists(CLANG):
+        pytest.skip("no host clang++")
+    out = tmp_path_factory.mktemp("host_block_mfma")
+    flags = ["-x", "c++", "-std=c++20", "-O1", "-fPIC", "-pthread", "-I", os.path.join(HERE, "host_block"), "-I", fta_build.INCLUDE, "-I", fta_build.CSRC]
+    srcs = [os.path.join(fta_build.CSRC, s) for s in SOURCES] + [os.path.join(HERE, "host_block", "stage1_mfma_host.cpp")]
+    procs, objs = [], []
+    for src in srcs:
+        obj = str(out / (os.path.basename(src) + ".o"))
+        level = ["-O0"] if src.endswith("stage1_mfma_host.cpp") else []     # twenty instantiations: half a minute to optimise
+        procs.append(subprocess.Popen([CLANG, *flags, *level, "-c", src, "-o", obj], stdout=subprocess.PIPE, stderr=subprocess.STDOUT))
+        objs.append(obj)
+    for proc in procs:
+        log = proc.communicate()[0]
+        assert proc.returncode == 0, log.decode()[-3000:]
+    path = str(out / "libfta_host_mfma.so")
+    subprocess.run([CLANG, "-shared", "-pthread", *objs, "-o", path], check=True, capture_output=True)
+    lib = C.CDLL(path)
+    for name in ("fta_decode", "fta_decode_stage1", "fta_decode_stage2"):
+        getattr(lib, name).argtypes = [C.POINTER(_lib.FtaArgs), C.c_void_p]
+    lib.fta_plan.argtypes = [C.POINTER(_lib.FtaArgs), C.c_int, C.POINTER(_lib.FtaPlanOut)]
+    assert lib.fta_abi_version() == _lib.ABI_VERSION
+    return lib
+
+
+def clamped(x, lens, tmax):
+    return dict(x, kv_seq_len=torch.tensor([min(max(t, 0), tmax) for t in lens]))
+
+
+@pytest.mark.parametrize("shape", [
+    # bsz hq hkv L  D    tmax dtype           lens         splits rows_per_wg
+    (2, 4, 2, 5, 64, 300, torch.bfloat16, [200, 77], 2, 128),        # 4 waves, rings of 2; ragged last tiles; one wave holds rows
+    (1, 8, 1, 20, 128, 512, torch.float16, [470], 1, 256),           # 8 waves pipelined, 8 tiles through rings of 3 and 5, 160 rows, straight to `out`
+    (2, 4, 1, 70, 64, 256, torch.bfloat16, [256, 64], 2, 256),       # 280 rows: two row blocks, the second nearly empty; two tree tiles; a split of whole tiles only
+    (1, 2, 2, 3, 256, 256, torch.float16, [100], 1, 128),            # head_dim 256
+    (3, 4, 2, 7, 128, 320, torch.bfloat16, [0, 999, -5], 3, 128),    # an empty cache, a length beyond the cache (clamped), a negative one (empty)
+    (2, 2, 2, 33, 128, 192, torch.float16, [65, 1], 2, 128),         # 33 rows: the second wave holds one row; one key in the cache
+])
+def test_whole_call(host_lib, shape):
+    bsz, hq, hkv, L, D, tmax, dtype, lens, splits, rows_per_wg = shape
+    x = make(11, bsz, hq, hkv, L, D, tmax, dtype, lens)
+    call = HostCall(host_lib, x, splits=splits, kernel=MFMA)
+    assert call.plan.kernel == MFMA and call.plan.rows_per_wg == rows_per_wg and not call.plan.mfma_loop
+    out = call.run()
+    assert torch.isfinite(out).all()
+    torch.testing.assert_close(out.float(), oracle(clamped(x, lens, tmax)), **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype,D", [(torch.bfloat16, 128), (torch.float16, 64)])
+def test_stage1_alone_fills_the_slots_the_oracle_predicts(host_lib, dtype, D):
+    """A cache far larger than the sequences: the kernel itself takes the chunk from the batch's longest sequence.
+    Every live slot against the oracle's partial of that split (the owner of a sequence's end also holds the tree
+    block); slots that a sequence does not reach stay untouched."""
+    lens, tmax, S = [700, 130, 0], 8192, 4
+    x = make(5, 3, 4, 2, 6, D, tmax, dtype, lens)
+    call = HostCall(host_lib, x, splits=S, kernel=MFMA)
+    assert call.plan.num_splits == S
+    chunk = call.plan.chunk_for(max(lens))
+    assert chunk < call.plan.chunk and chunk % 64 == 0
+    call.run("fta_decode_stage1")
+    assert torch.isnan(call.out).all()
+    for b, t_b in enumerate(lens):
+        parts = expected_partials(x, b, chunk, S)
+        assert len(parts) == live_splits(t_b, chunk, S)
+        for s, (o_ref, lse_ref) in enumerate(parts):
+            torch.testing.assert_close(call.lse[b, :, s], lse_ref, atol=2e-3, rtol=1e-3)
+            torch.testing.assert_close(call.mid[b, :, s], o_ref, **TOL[dtype])
+        for s in range(len(parts), S):
+            assert torch.isnan(call.mid[b, :, s]).all() and torch.isnan(call.lse[b, :, s]).all()
+    out = call.run("fta_decode_stage2")
+    torch.testing.assert_close(out.float(), oracle(x), **TOL[dtype])
+
+
+@pytest.mark.parametrize("rows_per_wg", [128, 256])
+def test_merge_inside_the_launch(host_lib, rows_per_wg):
+    """With counters the workgroup that finishes a (sequence, unit, row block) last merges the partials itself and
+    leaves the counters at zero; the result is that of the two-launch path bit for bit."""
+    hq, L = (4, 6) if rows_per_wg == 128 else (8, 20)
+    lens, tmax = [300, 64, 0], 320
+    x = make(13, 3, hq, 1, L, 128, tmax, torch.bfloat16, lens)
+    two = HostCall(host_lib, x, splits=3, kernel=MFMA)
+    assert two.plan.rows_per_wg == rows_per_wg
+    ref = two.run().clone()
+    one = HostCall(host_lib, x, splits=3, kernel=MFMA, counters=True)
+    assert one.plan.counter_elems > 0
+    out = one.run()                             # fta_decode launches stage 1 only
+    assert torch.isnan(one.mid[2]).all()        # (the empty sequence has one split and goes straight to `out`)
+    torch.testing.assert_close(out.float(), oracle(x), **TOL[torch.bfloat16])
+    assert torch.equal(out, ref)
+    assert (one.counters == 0).all()
+    out.fill_(float("nan"))
+    assert torch.equal(one.run(), ref)          # and again, on the counters it left
+
+
+def test_paged_caches_and_packed_mask(host_lib):
+    lens, tmax, page = [300, 33], 384, 16
+    x = make(7, 2, 4, 2, 6, 128, tmax, torch.float16, lens)
+    per_seq = tmax // page
+    g = torch.Generator().manual_seed(2)
+    perm = torch.randperm(2 * per_seq + 3, generator=g)[: 2 * per_seq].view(2, per_seq)
+    kp = torch.full((2 * per_seq + 3, 2, page, 128), float("nan"), dtype=torch.float16)
+    vp = torch.full_like(kp, float("nan"))
+    for b in range(2):
+        for pg in range(per_seq):
+            kp[perm[b, pg]] = x["k_cache"][b, :, pg * page:(pg + 1) * page]
+            vp[perm[b, pg]] = x["v_cache"][b, :, pg * page:(pg + 1) * page]
+    tables = torch.zeros(2, 96, dtype=torch.int32)             # a table four times wider than the sequences need
+    tables[:, :per_seq] = perm.to(torch.int32)
+    plain = HostCall(host_lib, x, splits=2, hint=tmax, kernel=MFMA).run().clone()
+    paged = HostCall(host_lib, x, splits=2, hint=tmax, tables=tables, pools=(kp, vp), mask=pack_mask(x["mask"]), kernel=MFMA).run()
+    torch.testing.assert_close(paged.float(), oracle(x), **TOL[torch.float16])
+    assert torch.equal(paged, plain)                           # where rows come from changes nothing of what is computed
+
+
+def test_paged_pipelined(host_lib):
+    """The 8-wave loop fetches the next tile's pages ahead of its barrier: pages of 64 keys (one per tile) and of
+    16 keys (the smallest the library takes), in a pool whose unused pages hold NaN."""
+    lens, tmax = [448], 512
+    x = make(17, 1, 8, 1, 20, 128, tmax, torch.bfloat16, lens)
+    ref = oracle(x)
+    for page in (64, 16):
+        n = tmax // page
+        perm = torch.randperm(n + 5, generator=torch.Generator().manual_seed(page))[:n]
+        kp = torch.full((n + 5, 1, page, 128), float("nan"), dtype=torch.bfloat16)
+        vp = torch.full_like(kp, float("nan"))
+        for pg in range(n):
+            kp[perm[pg]] = x["k_cache"][0, :, pg * page:(pg + 1) * page]
+            vp[perm[pg]] = x["v_cache"][0, :, pg * page:(pg + 1) * page]
+        tables = perm.to(torch.int32).view(1, n).contiguous()
+        call = HostCall(host_lib, x, splits=2, hint=tmax, tables=tables, pools=(kp, vp), kernel=MFMA)
+        assert call.plan.rows_per_wg == 256
+        torch.testing.assert_close(call.run().float(), ref, **TOL[torch.bfloat16])
+
+
+def test_peaked_logits_take_the_rescale_path(host_lib):
+    """Scores that grow along the sequence raise the running maximum in nearly every tile (the rescale of O that
+    is deferred behind the next P.V product), and a mask row that admits only the token itself."""
+    lens, tmax, D = [384], 384, 128
+    x = make(19, 1, 8, 1, 20, D, tmax, torch.float16, lens)
+    ramp = torch.linspace(0.2, 3.0, tmax).view(1, 1, tmax, 1)
+    x["k_cache"] = (x["q"][:, :1, :1, :].float() * ramp).to(torch.float16)       # keys ever more aligned with the first query row
+    call = HostCall(host_lib, x, splits=1, kernel=MFMA)
+    assert call.plan.rows_per_wg == 256
+    torch.testing.assert_close(call.run().float(), oracle(x), **TOL[torch.float16])
