@@ -35,9 +35,10 @@ def parse():
     ap.add_argument("--config", default="cfg3_gqa_8b_bf16", help="workload name (flash_tree_attn_amd.synthetic.CONFIGS)")
     ap.add_argument("--kv-sets", type=int, default=0, help="independent KV caches to rotate over (0 = enough for >1 GiB)")
     ap.add_argument("--splits", type=int, default=0, help="pin the split count (0 = heuristic)")
-    ap.add_argument("--kernel", default="auto", choices=["auto", "mfma", "mfma_wide", "shuffle"],
+    ap.add_argument("--kernel", default="auto", choices=["auto", "mfma", "mfma_wide", "mfma_split_keys", "shuffle"],
                     help="pin the stage-1 kernel (auto = the plan's choice); for comparing them on one workload. mfma_wide = the "
-                         "MFMA kernel with 64-row waves and the hand-scheduled half-tile loop (256-row units, contiguous caches)")
+                         "MFMA kernel with 64-row waves and the hand-scheduled half-tile loop (256-row units, contiguous caches); mfma_split_keys = "
+                         "the MFMA kernel with two waves per 32-row block, each taking half of a tile's keys (units of at most 64 rows)")
     ap.add_argument("--op", default="decode", choices=["decode", "append_kv"],
                     help="decode = the tree-attention call (the headline); append_kv = the accepted-path KV append that follows it")
     ap.add_argument("--accept", type=int, default=8, help="accepted tree rows per sequence for --op append_kv")
@@ -267,7 +268,7 @@ def main():
                 x["k_cache_paged"], x["v_cache_paged"], x["tables"] = kc, vc, tables
         calls.append(prepare(x["q"], kc, vc, x["current_k"], x["current_v"], mask_arg, x["kv_seq_len"], cfg.block_size,
                              None, None, None, None, x["sm_scale"], cfg.kv_group_num, _force_splits=args.splits,
-                             _force_kernel={"auto": -1, "mfma": _lib.KERNEL_MFMA, "mfma_wide": _lib.KERNEL_MFMA_WIDE, "shuffle": _lib.KERNEL_SHUFFLE}[args.kernel],
+                             _force_kernel={"auto": -1, "mfma": _lib.KERNEL_MFMA, "mfma_wide": _lib.KERNEL_MFMA_WIDE, "mfma_split_keys": _lib.KERNEL_MFMA_SPLIT_KEYS, "shuffle": _lib.KERNEL_SHUFFLE}[args.kernel],
                              block_tables=tables))
     if args.paged:   # the contiguous copies are no longer needed, except set 0 for the self-check
         x["k_caches"], x["v_caches"] = x["k_caches"][:1], x["v_caches"][:1]
@@ -335,7 +336,7 @@ def main():
                    "head_dim": cfg.head_dim, "q_len": cfg.q_len, "cache_len": cfg.cache_len, "lengths": cfg.lengths,
                    "block_size": cfg.block_size, "mask": "packed u64" if args.packed_mask else "additive f32",
                    "kv_layout": f"paged, {args.paged} positions per page, shuffled pool" if args.paged else "contiguous per sequence", "kv_sets_rotated": kv_sets, "num_splits": plan.num_splits,
-                   "chunk": plan.chunk, "chunk_for_these_lengths": plan.chunk_for(int(x["kv_seq_len"].max())), "stage1_kernel": ("mfma_wide" if plan.mfma_loop else "mfma") if plan.kernel == _lib.KERNEL_MFMA else "shuffle",
+                   "chunk": plan.chunk, "chunk_for_these_lengths": plan.chunk_for(int(x["kv_seq_len"].max())), "stage1_kernel": ("mfma", "mfma_wide", "mfma_split_keys")[plan.mfma_loop] if plan.kernel == _lib.KERNEL_MFMA else "shuffle",
                    "stage1_workgroups": plan.num_workgroups, "algorithmic_bytes": nbytes, "flops": nflops},
         "tflops": nflops / (ms * 1e-3) / 1e12,
         "roofline": {"bound": "hbm", "kernel": "stage1", "achieved": round(gbs_s1, 1), "peak": HBM_PEAK_GBS,

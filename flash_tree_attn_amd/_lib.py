@@ -11,7 +11,7 @@ ABI_VERSION = 3
 FTA_F32, FTA_F16, FTA_BF16 = 0, 1, 2
 FTA_I32, FTA_I64 = 0, 1
 MASK_ADDITIVE_F32, MASK_PACKED_U64 = 0, 1
-KERNEL_SHUFFLE, KERNEL_MFMA, KERNEL_MFMA_WIDE = 0, 1, 2
+KERNEL_SHUFFLE, KERNEL_MFMA, KERNEL_MFMA_WIDE, KERNEL_MFMA_SPLIT_KEYS = 0, 1, 2, 3
 
 EXPORTED_SYMBOLS = (
     "fta_abi_version", "fta_strerror", "fta_validate", "fta_plan", "fta_decode", "fta_decode_stage1",

@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 LIB_PATH = os.path.join(HERE, "libfta.so")
-SOURCES = ["fta_host.cpp", "stage1_shuffle.hip", "stage1_mfma.hip", "stage1_mfma_wide.hip", "stage2_merge.hip", "append_kv.hip"]
+SOURCES = ["fta_host.cpp", "stage1_shuffle.hip", "stage1_mfma.hip", "stage1_mfma_wide.hip", "stage1_mfma_splitkeys.hip", "stage2_merge.hip", "append_kv.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",

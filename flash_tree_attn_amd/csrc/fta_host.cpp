@@ -20,6 +20,7 @@ const EnvKnobs& env_knobs() {
     k.tree_tile_weight = -1;
     if (const char* e = std::getenv("FTA_TREE_TILE_WEIGHT")) k.tree_tile_weight = std::max(0, std::atoi(e));
     if (const char* e = std::getenv("FTA_WIDE_LOOP")) k.wide_loop = e[0] == '1';
+    if (const char* e = std::getenv("FTA_SPLIT_KEYS")) k.split_keys = e[0] == '1';
     return k;
   }();
   return knobs;
@@ -75,7 +76,7 @@ int validate(const fta_args& a) {
     return FTA_ERR_SHAPE;
   if (a.num_q_heads % a.num_kv_heads != 0) return FTA_ERR_SHAPE;
   if (a.cur_heads != a.num_kv_heads && a.cur_heads != a.num_q_heads) return FTA_ERR_SHAPE;
-  if (a.force_kernel < -1 || a.force_kernel > FTA_KERNEL_MFMA_WIDE) return FTA_ERR_UNSUPPORTED;
+  if (a.force_kernel < -1 || a.force_kernel > FTA_KERNEL_MFMA_SPLIT_KEYS) return FTA_ERR_UNSUPPORTED;
   // Paged caches with no capacity have no table entry to look up (the kernels clamp positions to cache_len - 1).
   if (a.block_table && a.cache_len == 0) return FTA_ERR_SHAPE;
 
@@ -107,7 +108,13 @@ int plan(const fta_args& a, int num_cus, fta_plan_out* out) {
     if (a.force_kernel != FTA_KERNEL_SHUFFLE && !mfma_eligible(a)) return FTA_ERR_UNSUPPORTED;
     kernel = a.force_kernel == FTA_KERNEL_SHUFFLE ? FTA_KERNEL_SHUFFLE : FTA_KERNEL_MFMA;
   }
-  const int rows_per_wg = kernel == FTA_KERNEL_MFMA ? mfma_rows_per_wg(rows, a.head_dim) : 16;
+  // Units of at most 64 rows, head_dim 64 / 128: two waves per 32-row block, each taking half of a tile's
+  // keys, so that all four waves of the workgroup compute (with 32-row waves, three or two of them would only
+  // request tiles). Opt-in (force_kernel or FTA_SPLIT_KEYS=1) until it has been timed.
+  const bool split_ok = kernel == FTA_KERNEL_MFMA && rows <= 64 && a.head_dim <= 128;
+  if (a.force_kernel == FTA_KERNEL_MFMA_SPLIT_KEYS && !split_ok) return FTA_ERR_UNSUPPORTED;
+  const bool split_keys = split_ok && (a.force_kernel == FTA_KERNEL_MFMA_SPLIT_KEYS || (a.force_kernel < 0 && env_knobs().split_keys));
+  const int rows_per_wg = kernel != FTA_KERNEL_MFMA ? 16 : split_keys ? 64 : mfma_rows_per_wg(rows, a.head_dim);
   // The 64-row-wave loop serves 256-row workgroups on contiguous caches, head_dim 64 / 128. It is
   // opt-in (force_kernel or FTA_WIDE_LOOP=1): at the headline shape it measures level with the
   // 8-wave loop, ahead of it on long chunks and behind it on short ones.
@@ -118,7 +125,7 @@ int plan(const fta_args& a, int num_cus, fta_plan_out* out) {
   // Workgroups one CU holds at a time (LDS- and register-bound, see the kernels): the
   // 128-row MFMA variant is built to share a CU with a second workgroup.
   // The shuffle kernel's workgroups (4 waves, ~40 KB of LDS) fit four to a CU.
-  const int wg_per_cu = kernel != FTA_KERNEL_MFMA ? 4 : (rows_per_wg == 128 && a.head_dim <= 128) ? 2 : 1;
+  const int wg_per_cu = kernel != FTA_KERNEL_MFMA ? 4 : (rows_per_wg <= 128 && a.head_dim <= 128) ? 2 : 1;
 
   const int64_t work_items = static_cast<int64_t>(a.bsz) * units * row_blocks;
   const int64_t t_cap = a.max_seq_len_hint > 0 ? std::min(a.max_seq_len_hint, a.cache_len) : a.cache_len;
@@ -227,7 +234,7 @@ int plan(const fta_args& a, int num_cus, fta_plan_out* out) {
   out->rows_per_wg = rows_per_wg;
   out->row_blocks = row_blocks;
   out->num_workgroups = static_cast<int32_t>(work_items * splits);
-  out->mfma_loop = wide ? 1 : 0;
+  out->mfma_loop = wide ? 1 : split_keys ? 2 : 0;
   out->counter_elems = (splits > 1 && kernel == FTA_KERNEL_MFMA && work_items <= 0x7fffffff) ? static_cast<int32_t>(work_items) : 0;
   // Merging inside stage 1 saves the second launch, but the last workgroup of a sequence
   // merges alone: that pays with two splits and one round of workgroups (short launches,
@@ -323,7 +330,7 @@ int decode_impl(const fta_args* args, void* hip_stream, int stages) {
   p.block_table = a.block_table;
   p.table_stride = a.block_table_stride;
   p.page_shift = a.page_size == 16 ? 4 : a.page_size == 32 ? 5 : a.page_size == 64 ? 6 : 7;
-  p.wide_loop = pl.mfma_loop;
+  p.wide_loop = pl.mfma_loop == 1;
   p.bsz = a.bsz; p.num_q_heads = a.num_q_heads; p.q_len = a.q_len; p.cache_len = a.cache_len;
   p.chunk = pl.chunk; p.num_splits = pl.num_splits;
   for (int i = 0; i < FTA_LEN_BUCKETS; ++i) {

@@ -65,18 +65,20 @@ struct KernelParams {
 int launch_stage1_shuffle(const KernelParams& p, int dtype, int head_dim, void* stream);
 int launch_stage1_mfma(const KernelParams& p, int dtype, int head_dim, void* stream);
 int launch_stage1_mfma_wide(const KernelParams& p, int dtype, int head_dim, void* stream);   // 256-row workgroups of 64-row waves
+int launch_stage1_mfma_splitkeys(const KernelParams& p, int dtype, int head_dim, void* stream);   // 64-row workgroups, two waves per row block
 int launch_stage2_merge(const KernelParams& p, int dtype, int head_dim, void* stream);
 
 // Rows one MFMA workgroup holds for a unit of `rows` query rows (host + device agree on it).
 int mfma_rows_per_wg(int rows, int head_dim);
 
 // Tuning knobs from the environment, read once per process (comparison runs and tests only):
-// FTA_ROWS_PER_WG=128, FTA_FORCE_SPLITS=n, FTA_TREE_TILE_WEIGHT=n, FTA_WIDE_LOOP=1.
+// FTA_ROWS_PER_WG=128, FTA_FORCE_SPLITS=n, FTA_TREE_TILE_WEIGHT=n, FTA_WIDE_LOOP=1, FTA_SPLIT_KEYS=1.
 struct EnvKnobs {
   bool rows_128;
   int force_splits;      // 0 = none
   int tree_tile_weight;  // < 0 = default
   bool wide_loop;
+  bool split_keys;
 };
 const EnvKnobs& env_knobs();
 

@@ -22,6 +22,8 @@ int launch_t(const KernelParams& p, int head_dim, hipStream_t stream) {
     if (head_dim == 128) return launch<T, 128, 1, 4, 2, kPlain, PAGED>(p, stream);
     if (head_dim == 64) return launch<T, 64, 1, 4, 2, kPlain, PAGED>(p, stream);
     if (head_dim == 256) return launch<T, 256, 1, 4, 2, kPlain, PAGED>(p, stream);   // 132 KB of rings: one workgroup per CU
+  } else if (p.rows_per_wg == 64) {   // 4 waves, two per row block, each half of a tile's keys (stage1_mfma_splitkeys.hip)
+    return launch_stage1_mfma_splitkeys(p, dtype_of(T{}), head_dim, stream);
   }
   return FTA_ERR_UNSUPPORTED;
 }

@@ -83,6 +83,7 @@ namespace {
 constexpr int kPlain = 0;       // 4 waves x 32 rows, one tile at a time, short rings, two workgroups per CU
 constexpr int kPipelined = 1;   // 8 waves x 32 rows, software pipeline over whole tiles
 constexpr int kWide = 2;        // 4 waves x 64 rows, software pipeline over half tiles, one wave per SIMD
+constexpr int kSplitKeys = 3;   // 4 waves, 64 rows: like kPlain, but two waves share a 32-row block, each taking 32 of a tile's 64 keys
 
 // NSK >= 2: K of tile t+1 is read during iteration t and must have been requested an
 // iteration earlier.
@@ -96,6 +97,8 @@ stage1_mfma_kernel(const KernelParams p) {
   static_assert(NSK >= 2, "K ring too shallow");
   constexpr bool PIPE = MODE == kPipelined;
   constexpr bool WIDE = MODE == kWide;
+  constexpr bool KSPLIT = MODE == kSplitKeys;
+  static_assert(!KSPLIT || (QB == 1 && NW % 2 == 0), "key halves are written for one row block per wave and pairs of waves");
   static_assert(!WIDE || QB == 2, "the half-tile pipeline is written for two row blocks per wave");
   // V ring: the pipelined loop reads V of a tile one iteration (a whole tile) after its K,
   // the half-tile pipeline half a tile after
@@ -107,7 +110,7 @@ stage1_mfma_kernel(const KernelParams p) {
   static_assert(TL::kBlocks % NW == 0 && kLoadsPerTensor >= 1, "loader mapping");
   constexpr int kLoadsPerTile = 2 * kLoadsPerTensor;
   constexpr int kRowsPerWave = 32 * QB;
-  constexpr int kRowsPerWg = NW * kRowsPerWave;
+  constexpr int kRowsPerWg = (KSPLIT ? NW / 2 : NW) * kRowsPerWave;
   constexpr int kVRing = NSK * TL::kTileBytes;       // byte offset of the V ring
 
   FTA_DYNAMIC_LDS(smem);
@@ -130,7 +133,9 @@ stage1_mfma_kernel(const KernelParams p) {
   const int head0 = w.unit * p.heads_per_unit;
   const int cache_head = head0 / p.kv_group;
   const int cur_head = head0 / p.cur_group;
-  const int wave_row0 = w.row_block * kRowsPerWg + wave * kRowsPerWave;
+  // kSplitKeys: waves 2r and 2r+1 hold the same 32 rows; wave 2r+h takes keys 32h .. 32h+31 of every tile
+  const int kb_own = KSPLIT ? (wave & 1) : 0;
+  const int wave_row0 = w.row_block * kRowsPerWg + (KSPLIT ? wave >> 1 : wave) * kRowsPerWave;
   const bool wave_active = wave_row0 < p.rows;
   const float c = p.scale_log2;
 
@@ -667,6 +672,144 @@ stage1_mfma_kernel(const KernelParams p) {
     }
   };
 
+  // ---- key halves (MODE == kSplitKeys) -----------------------------------------------
+  // Units of a few rows fill one or two waves of a 4-wave workgroup; the others would only
+  // request tiles. Here two waves hold the same 32 rows and each takes 32 of a tile's 64 keys
+  // (key block kb_own): the same fragments, layouts and steps as the plain loop, half of
+  // them per wave, with an online-softmax state of its own that is merged with its
+  // partner's through LDS after the last tile (the merge of flash_tree_attn.py:185-211 in
+  // its unnormalised form).
+  auto qk_half = [&](int t, f32x16& s) __attribute__((always_inline)) {
+    const uint32_t ka = k_rd + (t % NSK) * TL::kTileBytes + kb_own * kKbOff;
+    u32x4 kf[KS];
+    static_for<0, kPF>([&](auto f) { kf[f] = lds_read_b128<f * kKsOff>(ka); });
+    static_for<0, KS>([&](auto f) {
+      constexpr int kNewer = (KS - 1 - f) < (kPF - 1) ? (KS - 1 - f) : (kPF - 1);
+      wait_lgkm<kNewer>(kf[f]);
+      const Vec8 a = __builtin_bit_cast(Vec8, kf[f]);
+      if constexpr (f == 0) {
+        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        s = M::mma(a, qf[0][f], zero);
+      } else {
+        s = M::mma(a, qf[0][f], s);
+      }
+      if constexpr (f + kPF < KS) kf[f + kPF] = lds_read_b128<(f + kPF) * kKsOff>(ka);
+    });
+  };
+  auto pv_half = [&](int t, const Vec8 (&pf)[2]) __attribute__((always_inline)) {
+    constexpr int kFrags = 2 * DB;   // two groups of 16 keys x DB blocks of head_dim
+    static_assert(KS >= kPF && kFrags >= kPF, "fragment queues deeper than the streams");
+    const uint32_t va = v_rd + (t % NSV) * TL::kTileBytes + kb_own * 2 * kVRowsOff16;
+    u32x2 vlo[kFrags], vhi[kFrags];
+    auto issue_v = [&](auto g) __attribute__((always_inline)) {
+      constexpr int kOff = (g / DB) * kVRowsOff16 + (g % DB) * 4 * TL::kChunkStride;
+      vlo[g] = lds_read_tr16_b64<kOff>(va);
+      vhi[g] = lds_read_tr16_b64<kOff + kVRowsOff8>(va);
+    };
+    static_for<0, kPF>(issue_v);
+    static_for<0, kFrags>([&](auto g) {
+      constexpr int kNewer = (kFrags - 1 - g) < (kPF - 1) ? (kFrags - 1 - g) : (kPF - 1);
+      wait_lgkm<2 * kNewer>(vlo[g], vhi[g]);
+      const s16x8 both = __builtin_shufflevector(__builtin_bit_cast(s16x4, vlo[g]), __builtin_bit_cast(s16x4, vhi[g]), 0, 1, 2, 3, 4, 5, 6, 7);
+      o[g % DB][0] = M::mma(__builtin_bit_cast(Vec8, both), pf[g / DB], o[g % DB][0]);
+      if constexpr (g + kPF < kFrags) issue_v(std::integral_constant<int, g + kPF>{});
+    });
+  };
+  // Additive mask values of the wave's 32 tree keys from key0 on (load_mask for one key block).
+  auto load_mask_half = [&](int key0, float (&mv)[16]) __attribute__((always_inline)) {
+    const int64_t mstart = b * p.mask_stride[0] + row_head[0] * p.mask_stride[1] + row_i[0] * p.mask_stride[2];
+    if (p.mask_packed) {
+      const uint64_t wbits = static_cast<const uint64_t*>(p.mask)[mstart + (key0 >> 6)];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int j = (key0 & 63) + (r >> 2) * 8 + 4 * lh + (r & 3);
+        mv[r] = (wbits >> j) & 1 ? 0.f : neg_inf();
+      }
+      return;
+    }
+    const float* mrow = static_cast<const float*>(p.mask) + mstart;
+#pragma unroll
+    for (int rg = 0; rg < 4; ++rg) {
+      const int j0 = key0 + rg * 8 + 4 * lh;
+      if (p.mask_vec4 && j0 + 3 < L) {
+        const f32x4 v4 = *reinterpret_cast<const f32x4*>(mrow + j0);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) mv[rg * 4 + e] = v4[e];
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) mv[rg * 4 + e] = mrow[min(j0 + e, L - 1)];
+      }
+    }
+  };
+  // softmax_tile for one key block: scores of 32 keys in `s`, P^T of its two 16-key groups out in `pf`.
+  auto softmax_half = [&](auto masked_c, f32x16& s, Vec8 (&pf)[2], bool tree, int key0, int key_lim, const float (&mv)[16]) __attribute__((always_inline)) {
+    constexpr bool MASKED = decltype(masked_c)::value;
+    const float m_old = m_run[0];
+    if (MASKED) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int j = key0 + (r >> 2) * 8 + 4 * lh + (r & 3);
+        float sv = s[r] * c;
+        if (tree) sv = __builtin_fmaf(mv[r], kLog2e, sv);
+        s[r] = j < key_lim ? sv : neg_inf();
+      }
+    }
+    float mx0 = s[0], mx1 = s[1];
+#pragma unroll
+    for (int r = 2; r < 16; r += 2) {
+      mx0 = fmaxf(mx0, s[r]);
+      mx1 = fmaxf(mx1, s[r + 1]);
+    }
+    const float mx = half_swap_max(fmaxf(mx0, mx1), lh);
+    const float m_new = fmaxf(m_old, MASKED ? mx : mx * c);
+    const float m_use = (MASKED && m_new == neg_inf()) ? 0.f : m_new;
+    const float alpha = fast_exp2(m_old - m_use);
+    float ps0 = 0.f, ps1 = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; r += 2) {
+      const float p0 = MASKED ? fast_exp2(s[r] - m_use) : fast_exp2(__builtin_fmaf(s[r], c, -m_use));
+      const float p1 = MASKED ? fast_exp2(s[r + 1] - m_use) : fast_exp2(__builtin_fmaf(s[r + 1], c, -m_use));
+      s[r] = p0;
+      s[r + 1] = p1;
+      ps0 += p0;
+      ps1 += p1;
+    }
+    l_run[0] = l_run[0] * alpha + (ps0 + ps1);
+    m_run[0] = m_new;
+    alpha_pending[0] = alpha;
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      Vec8 pk;
+#pragma unroll
+      for (int e = 0; e < 8; e += 2) {
+        const f32x2 pv = {s[kk * 8 + e], s[kk * 8 + e + 1]};
+        const auto pr = __builtin_convertvector(pv, typename M::Vec2);
+        pk[e] = pr[0];
+        pk[e + 1] = pr[1];
+        if (MASKED) {  // keep the rounding residue for the compensating product
+          s[kk * 8 + e] = pv[0] - static_cast<float>(pr[0]);
+          s[kk * 8 + e + 1] = pv[1] - static_cast<float>(pr[1]);
+        }
+      }
+      pf[kk] = pk;
+    }
+    rescale_pending = wave_any(m_new > m_old);
+  };
+  auto pv_half_with_residue = [&](int tile, bool masked_tile, const f32x16& res, Vec8 (&pf)[2]) __attribute__((always_inline)) {
+    apply_rescale();
+    pv_half(tile, pf);
+    if (masked_tile) {
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) {
+        Vec8 pk;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) pk[e] = static_cast<T>(res[kk * 8 + e]);
+        pf[kk] = pk;
+      }
+      pv_half(tile, pf);
+    }
+  };
+
 
   // ---- the half-tile pipeline (MODE == kWide) ----------------------------------------
   // A wave holds 64 query rows (two row blocks), so every K or V fragment it reads from LDS
@@ -773,6 +916,52 @@ stage1_mfma_kernel(const KernelParams p) {
       pv_with_residue(t, masked, sB);
     }
     if (!wave_active) return;
+  } else if constexpr (KSPLIT) {
+    f32x16 s_half;
+    Vec8 p_half[2];
+    float mask_half[16];
+    for (int t = 0; t < ntiles; ++t) {
+      sync_point(t, t, t, ntiles);
+      if (!wave_active) continue;
+      const bool tree = t < tree_tiles;
+      const bool masked = tree || t - c0 >= full_tiles;
+      const int key0 = (tree ? t * kKeyTile : kv_start + (t - c0) * kKeyTile) + 32 * kb_own;
+      if (tree) load_mask_half(key0, mask_half);   // in flight while the scores are computed
+      qk_half(t, s_half);
+      if (masked) softmax_half(std::true_type{}, s_half, p_half, tree, key0, tree ? L : kv_end, mask_half);
+      else softmax_half(std::false_type{}, s_half, p_half, false, key0, kv_end, mask_half);
+      pv_half_with_residue(t, masked, s_half, p_half);
+    }
+    // The two waves of a row block merge their states: the wave of the upper key block parks
+    // m, l and O in LDS (the rings are idle: every tile has landed and been read once all
+    // waves are past the first barrier), the wave of the lower one folds them into its own
+    // and goes on to the epilogue. Lane-major layout: word k of lane i at (k * 64 + i).
+    constexpr int kStateWords = 2 + 16 * DB;
+    static_assert((NW / 2) * kStateWords * 64 * 4 <= 2 * NSK * TL::kTileBytes, "the parked states fit the rings");
+    float* park = reinterpret_cast<float*>(smem) + (wave >> 1) * kStateWords * 64 + lane;
+    __syncthreads();
+    if (kb_own == 1 && wave_active) {
+      park[0] = m_run[0];
+      park[64] = l_run[0];
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) park[(2 + db * 16 + r) * 64] = o[db][0][r];
+    }
+    __syncthreads();
+    if (kb_own == 1 || !wave_active) return;
+    {
+      const float m_other = park[0], l_other = park[64];
+      const float m_both = fmaxf(m_run[0], m_other);
+      const float m_use = m_both == neg_inf() ? 0.f : m_both;
+      const float a_own = fast_exp2(m_run[0] - m_use), a_other = fast_exp2(m_other - m_use);
+      l_run[0] = l_run[0] * a_own + l_other * a_other;
+      m_run[0] = m_both;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[db][0][r] = o[db][0][r] * a_own + park[(2 + db * 16 + r) * 64] * a_other;
+    }
   } else if constexpr (WIDE) {
     constexpr std::integral_constant<int, 0> h0{};
     constexpr std::integral_constant<int, 1> h1{};
@@ -1079,7 +1268,7 @@ stage1_mfma_kernel(const KernelParams p) {
 template <typename T, int D, int QB, int NW, int NS, int MODE, bool PAGED>
 int launch(const KernelParams& p, hipStream_t stream) {
   // K ring of NS stages + V ring of NS (+ 2 pipelined, + 1 half-tile pipeline)
-  constexpr int kSmem = (MODE == kPipelined ? 2 * NS + 2 : MODE == kWide ? 2 * NS + 1 : 2 * NS) * TileLayout<D>::kTileBytes;
+  constexpr int kSmem = (MODE == kPipelined ? 2 * NS + 2 : MODE == kWide ? 2 * NS + 1 : 2 * NS) * TileLayout<D>::kTileBytes;   // kPlain, kSplitKeys: 2 * NS
   static_assert(kSmem + 3 * 1024 <= 160 * 1024, "LDS budget (rings + the static arrays of item_by_order)");
   auto kern = stage1_mfma_kernel<T, D, QB, NW, NS, MODE, PAGED>;
   if (kSmem > 64 * 1024) {
@@ -1095,6 +1284,7 @@ int launch(const KernelParams& p, hipStream_t stream) {
   }
   const int64_t grid = static_cast<int64_t>(p.bsz) * p.units * p.row_blocks * p.num_splits;
   if (grid <= 0 || grid > 0x7fffffffLL) return FTA_ERR_SHAPE;
+  if (p.rows_per_wg != (MODE == kSplitKeys ? NW / 2 : NW) * 32 * QB) return FTA_ERR_SHAPE;   // the plan's row blocks are this kernel's
   return launch_checked(kern, dim3(static_cast<unsigned>(grid)), dim3(NW * 64), kSmem, stream, p);
 }
 

@@ -51,9 +51,13 @@ typedef enum fta_mask_kind {
 typedef enum fta_kernel {
   FTA_KERNEL_SHUFFLE = 0,  /* wavefront-shuffle reductions: any dtype / head_dim / q_len / sign of sm_scale */
   FTA_KERNEL_MFMA = 1,     /* MFMA tiles: f16/bf16, head_dim 64/128/256, sm_scale > 0; any number of rows */
-  FTA_KERNEL_MFMA_WIDE = 2 /* only as fta_args.force_kernel: the MFMA kernel with 64 query rows per wave and the
+  FTA_KERNEL_MFMA_WIDE = 2,/* only as fta_args.force_kernel: the MFMA kernel with 64 query rows per wave and the
                               hand-scheduled half-tile loop, for units of more than 128 rows on contiguous caches,
                               head_dim 64/128. A plan reports it as FTA_KERNEL_MFMA with mfma_loop = 1. */
+  FTA_KERNEL_MFMA_SPLIT_KEYS = 3 /* only as fta_args.force_kernel: the MFMA kernel for units of at most 64 query rows,
+                              head_dim 64/128, with two waves per 32-row block that each take half of a tile's keys
+                              (all four waves of a workgroup compute). A plan reports it as FTA_KERNEL_MFMA with
+                              rows_per_wg = 64 and mfma_loop = 2. */
 } fta_kernel;
 
 /*
@@ -157,7 +161,8 @@ typedef struct fta_plan_out {
   int32_t single_launch;  /* 1 where the single-launch path is expected to be the faster one (two splits, one
                              round of workgroups: the last workgroup of a sequence merges alone, which does
                              not pay for more) */
-  int32_t mfma_loop;      /* MFMA kernel, 256-row workgroups: 0 = 8 waves x 32 rows, 1 = 4 waves x 64 rows (half-tile loop) */
+  int32_t mfma_loop;      /* MFMA kernel: 0 = 32-row waves (4 per 128-row workgroup, 8 per 256-row one), 1 = 256-row workgroups of
+                             4 waves x 64 rows (half-tile loop), 2 = 64-row workgroups, two waves per 32-row block (key halves) */
   int64_t mid_o_elems;    /* float32 elements a dense mid_o for this plan needs */
   int64_t mid_lse_elems;
   /* Keys per split by the batch's longest sequence: the kernels read the lengths, find the first i

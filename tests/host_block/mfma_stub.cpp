@@ -3,4 +3,5 @@
 namespace fta {
 int launch_stage1_mfma(const KernelParams&, int, int, void*) { return FTA_ERR_UNSUPPORTED; }
 int launch_stage1_mfma_wide(const KernelParams&, int, int, void*) { return FTA_ERR_UNSUPPORTED; }
+int launch_stage1_mfma_splitkeys(const KernelParams&, int, int, void*) { return FTA_ERR_UNSUPPORTED; }
 }  // namespace fta

@@ -1,10 +1,12 @@
 // The MFMA stage-1 kernel's translation unit for the host-thread harness: the product source, with the
 // instruction wrappers of gfx950_ops.h replaced by the stand-ins of gfx950_ops_host.h (which must come
-// first: it claims the include guards). The 64-row-wave instantiations are assembly and stay out.
+// first: it claims the include guards), key-halves instantiations included. The 64-row-wave instantiations are
+// assembly and stay out.
 #include "fta_device.h"
 #include "gfx950_ops_host.h"
 
 #include "stage1_mfma.hip"
+#include "stage1_mfma_splitkeys.hip"
 
 namespace fta {
 int launch_stage1_mfma_wide(const KernelParams&, int, int, void*) { return FTA_ERR_UNSUPPORTED; }

@@ -292,12 +292,33 @@ def test_plan_of_the_64_row_wave_loop(fta_lib):
     a.k_stride[0] = a.v_stride[0] = 8 * 128 * 128
     a.k_stride[1] = a.v_stride[1] = 128 * 128
     assert fta_lib.fta_validate(C.byref(a)) == 0 and plan(fta_lib, a)[0] == -9
+
     a.force_kernel = -1
     st, pl = plan(fta_lib, a)
     assert st == 0 and pl.rows_per_wg == 256 and pl.mfma_loop == 0
     # a paged cache of no positions has no pages to name: rejected as a shape error
     a.cache_len = a.v_cache_len = 0
     assert fta_lib.fta_validate(C.byref(a)) == -7
+
+
+def test_plan_reports_key_halves_only_when_asked_and_refuses_them_where_they_do_not_exist(fta_lib):
+    """FTA_KERNEL_MFMA_SPLIT_KEYS: units of at most 64 rows, head_dim 64 / 128, any cache layout. Reported as the MFMA
+    kernel with 64-row workgroups and mfma_loop = 2; the cut is the 4-wave variant's (same cost model)."""
+    small = dict(num_q_heads=32, num_kv_heads=32, cur_heads=32, q_len=26, dtype=_lib.FTA_F16, force_kernel=_lib.KERNEL_MFMA_SPLIT_KEYS)
+    st, pl = plan(fta_lib, base_args(**small))
+    assert st == 0 and pl.kernel == _lib.KERNEL_MFMA and (pl.rows_per_wg, pl.row_blocks, pl.mfma_loop) == (64, 1, 2)
+    st, plain = plan(fta_lib, base_args(**{**small, "force_kernel": _lib.KERNEL_MFMA}))
+    assert st == 0 and (plain.rows_per_wg, plain.mfma_loop) == (128, 0)
+    assert (pl.num_splits, pl.chunk, pl.num_workgroups) == (plain.num_splits, plain.chunk, plain.num_workgroups)
+    if not os.environ.get("FTA_SPLIT_KEYS"):
+        st, auto = plan(fta_lib, base_args(**{**small, "force_kernel": -1}))
+        assert st == 0 and (auto.rows_per_wg, auto.mfma_loop) == (128, 0)
+    st, pl = plan(fta_lib, base_args(**{**small, "num_kv_heads": 8, "cur_heads": 8, "q_len": 16}))     # GQA 4 x 16 = 64 rows
+    assert st == 0 and pl.rows_per_wg == 64
+    assert plan(fta_lib, base_args(**{**small, "num_kv_heads": 8, "cur_heads": 8, "q_len": 17}))[0] == -9   # 68 rows
+    assert plan(fta_lib, base_args(**{**small, "head_dim": 256}))[0] == -9
+    assert plan(fta_lib, base_args(**{**small, "dtype": _lib.FTA_F32}))[0] == -9
+    assert plan(fta_lib, base_args(**{**small, "force_kernel": 4}))[0] == -9
 
 
 def test_python_wrapper_rejects_cpu_tensors():

@@ -178,3 +178,70 @@ def test_peaked_logits_take_the_rescale_path(host_lib):
     call = HostCall(host_lib, x, splits=1, kernel=MFMA)
     assert call.plan.rows_per_wg == 256
     torch.testing.assert_close(call.run().float(), oracle(x), **TOL[torch.float16])
+
+
+# ---- key halves: units of at most 64 rows, two waves per 32-row block ---------------------------------------------
+SPLIT_KEYS = _lib.KERNEL_MFMA_SPLIT_KEYS
+
+
+@pytest.mark.parametrize("shape", [
+    # bsz hq hkv L  D    tmax dtype           lens           splits
+    (2, 4, 2, 5, 64, 300, torch.bfloat16, [200, 77], 2),          # 10 rows: one pair of waves computes; ragged last tiles
+    (3, 4, 4, 26, 128, 320, torch.float16, [300, 64, 0], 3),      # 26 rows per head (MHA); an empty cache; a whole-tile split
+    (2, 4, 1, 16, 128, 256, torch.bfloat16, [256, 31], 2),        # 64 rows: both pairs compute; fewer keys than half a tile
+    (2, 8, 2, 1, 128, 256, torch.bfloat16, [256, 100], 2),        # plain decode, 4 rows
+    (1, 2, 1, 20, 64, 192, torch.float16, [33], 1),               # 40 rows: the second pair holds 8; one key in the upper half of a tile; straight to `out`
+    (2, 2, 2, 40, 64, 128, torch.bfloat16, [999, -5], 2),         # a tree whose second half tile is partly filled; clamped and negative lengths
+])
+def test_key_halves_whole_call(host_lib, shape):
+    bsz, hq, hkv, L, D, tmax, dtype, lens, splits = shape
+    x = make(23, bsz, hq, hkv, L, D, tmax, dtype, lens)
+    call = HostCall(host_lib, x, splits=splits, kernel=SPLIT_KEYS)
+    assert call.plan.kernel == MFMA and call.plan.rows_per_wg == 64 and call.plan.mfma_loop == 2 and call.plan.row_blocks == 1
+    out = call.run()
+    assert torch.isfinite(out).all()
+    torch.testing.assert_close(out.float(), oracle(clamped(x, lens, tmax)), **TOL[dtype])
+
+
+def test_key_halves_partials_counters_and_pages(host_lib):
+    """The partial of every live split (the two waves' states merged before the epilogue), then the same call with the
+    merge inside the launch, then on paged caches with the packed mask (bit-equal to the contiguous call)."""
+    lens, tmax, S, page = [500, 130, 0], 2048, 4, 16
+    x = make(29, 3, 4, 2, 12, 128, tmax, torch.bfloat16, lens)
+    call = HostCall(host_lib, x, splits=S, kernel=SPLIT_KEYS)
+    chunk = call.plan.chunk_for(max(lens))
+    assert call.plan.num_splits == S and chunk < call.plan.chunk
+    call.run("fta_decode_stage1")
+    for b, t_b in enumerate(lens):
+        parts = expected_partials(x, b, chunk, S)
+        for s, (o_ref, lse_ref) in enumerate(parts):
+            torch.testing.assert_close(call.lse[b, :, s], lse_ref, atol=2e-3, rtol=1e-3)
+            torch.testing.assert_close(call.mid[b, :, s], o_ref, **TOL[torch.bfloat16])
+        for s in range(len(parts), S):
+            assert torch.isnan(call.mid[b, :, s]).all() and torch.isnan(call.lse[b, :, s]).all()
+    ref = call.run("fta_decode_stage2").clone()
+    torch.testing.assert_close(ref.float(), oracle(x), **TOL[torch.bfloat16])
+    fused = HostCall(host_lib, x, splits=S, kernel=SPLIT_KEYS, counters=True)
+    out = fused.run()                                          # sums the four partials in another order: equal to the last bit or two
+    torch.testing.assert_close(out.float(), ref.float(), atol=1e-3, rtol=8e-3)
+    assert (out == ref).float().mean() > 0.98 and (fused.counters == 0).all()
+    per_seq = 512 // page                                      # pages for the first 512 positions only: nothing beyond is read
+    perm = torch.randperm(3 * per_seq, generator=torch.Generator().manual_seed(3)).view(3, per_seq)
+    kp = torch.full((3 * per_seq, 2, page, 128), float("nan"), dtype=torch.bfloat16)
+    vp = torch.full_like(kp, float("nan"))
+    for b in range(3):
+        for pg in range(per_seq):
+            kp[perm[b, pg]] = x["k_cache"][b, :, pg * page:(pg + 1) * page]
+            vp[perm[b, pg]] = x["v_cache"][b, :, pg * page:(pg + 1) * page]
+    tables = torch.zeros(3, tmax // page, dtype=torch.int32)
+    tables[:, :per_seq] = perm.to(torch.int32)
+    paged = HostCall(host_lib, x, splits=S, tables=tables, pools=(kp, vp), mask=pack_mask(x["mask"]), kernel=SPLIT_KEYS)
+    assert paged.plan.chunk_for(max(lens)) == chunk
+    assert torch.equal(paged.run(), ref)
+
+
+def test_key_halves_are_refused_where_they_do_not_exist(host_lib):
+    for hq, L, D in ((4, 20, 128), (2, 3, 256)):               # 80 rows per unit; head_dim 256
+        x = make(1, 1, hq, 1, L, D, 64, torch.float16, [64])
+        with pytest.raises(AssertionError):
+            HostCall(host_lib, x, kernel=SPLIT_KEYS)

@@ -2,8 +2,8 @@
 undefined-behaviour and thread sanitizers (GPU sanitizers do not exist on the target; host code is where
 they run). tests/host_block/sanitize_main.cpp calls fta_plan / fta_decode on buffers of exactly their size
 (contiguous and paged caches, ragged tiles, empty and over-long sequences, additive and packed masks; fp32
-through the shuffle kernel, bf16 through the MFMA kernel in its 4-wave, 8-wave pipelined and head_dim 256
-forms, with and without the merge inside the launch) and checks the results against a plain
+through the shuffle kernel, bf16 through the MFMA kernel in its 4-wave, 8-wave pipelined, head_dim 256 and
+key-halves forms, with and without the merge inside the launch) and checks the results against a plain
 double-precision attention.
   * address / undefined: a read or write one element past a tensor, a page, the scratch, an LDS array (the
     MFMA kernel's LDS addresses are checked against the launch's LDS size by the stand-ins themselves);
@@ -49,4 +49,4 @@ def test_host_build_is_clean_under(sanitize, tmp_path):
     for sign in ("AddressSanitizer", "runtime error", "data race", "ThreadSanitizer", "FAILED"):
         assert sign not in text, text[-3000:]
     assert r.returncode == 0 and text.strip().endswith("clean"), text[-2000:]
-    assert text.count("bf16/mfma") == 5, text[-2000:]
+    assert text.count("bf16/mfma") == 7, text[-2000:]

@@ -22,7 +22,7 @@ import pytest
 
 from flash_tree_attn_amd import build as fta_build
 
-UNITS = ["stage1_mfma.hip", "stage1_mfma_wide.hip"]
+UNITS = ["stage1_mfma.hip", "stage1_mfma_wide.hip", "stage1_mfma_splitkeys.hip"]
 
 
 def _generator():
@@ -43,7 +43,7 @@ def kernels():
             cmd = [fta_build.HIPCC, *fta_build.FLAGS, "--cuda-device-only", "-S", "-x", "hip", os.path.join(fta_build.CSRC, src), "-o", out]
             subprocess.run(cmd, check=True, capture_output=True)
             return open(out).read()
-        with ThreadPoolExecutor(max_workers=2) as pool:
+        with ThreadPoolExecutor(max_workers=3) as pool:
             texts = list(pool.map(compile_unit, UNITS))
     found = {}
     for text in texts:
@@ -54,8 +54,8 @@ def kernels():
         for m in re.finditer(r"^(_ZN3fta\S*stage1_mfma_kernel[^:\s]*):[^\n]*\n(.*?)^\.Lfunc_end", text, flags=re.S | re.M):
             lines = [l.strip() if l.strip().startswith(";;#ASM") else l.split(";")[0].strip() for l in m.group(2).split("\n")]
             found[m.group(1)] = ([l for l in lines if l and not l.startswith(".") and not l.endswith(":")], meta[m.group(1)])
-    # 2 dtypes x paged/contiguous x (pipelined D 128, 64 + plain D 128, 64, 256) + 2 dtypes x wide D 128, 64
-    assert len(found) == 2 * 2 * 5 + 2 * 2, sorted(found)
+    # 2 dtypes x paged/contiguous x (pipelined D 128, 64 + plain D 128, 64, 256 + key halves D 128, 64) + 2 dtypes x wide D 128, 64
+    assert len(found) == 2 * 2 * 7 + 2 * 2, sorted(found)
     return found
 
 
@@ -131,7 +131,7 @@ def touches_of_in_flight_lds_reads(ins):
 def test_registers_of_in_flight_lds_reads_are_left_alone(kernels):
     for name, (ins, _) in kernels.items():
         problems, reads = touches_of_in_flight_lds_reads(ins)
-        assert reads >= 32, (name, reads)            # every variant reads its K and V fragments this way
+        assert reads >= (20 if "Li3ELb" in name else 32), (name, reads)   # every variant reads its K and V fragments this way (key halves: half as many)
         assert not problems, (name, problems[:3])
     # the check sees what it is meant to see: a copy of a destination right behind its read is reported
     name, (ins, _) = next(iter(kernels.items()))

@@ -8,6 +8,7 @@ one-call path has:
   (flash_tree_attn.py:174-211), with sequences that fill fewer slots than the grid has;
 * caches much larger than the sequences in them (the cut must follow the lengths);
 * the 64-row-wave MFMA loop, which only runs when asked for;
+* the key-halves form of the MFMA kernel for small units, which only runs when asked for;
 * head_dim 256 through the merge inside stage 1 and on paged caches;
 * one sequence x two heads of the headline workload against the fp64 oracle on the CPU;
 * the largest error of each benchmark configuration as a share of the tolerance.
@@ -274,6 +275,45 @@ def test_64_row_wave_loop_at_headline_size():
     pc = prepare(x, _force_kernel=_lib.KERNEL_MFMA_WIDE)
     assert pc.plan.mfma_loop == 1
     check(pc.run(), oracle(x), cfg.dtype)
+
+
+# ---------------------------------------------------------------- key halves: small units, two waves per 32-row block
+KEY_HALVES_CASES = [
+    # name                               bsz hq hkv  L   D    T     lens                 splits dtype
+    ("26 rows, MHA, ragged", 4, 8, 8, 26, 128, 4096, [4096, 1000, 333, 0], 4, torch.float16),
+    ("64 rows, GQA 4 x 16", 2, 8, 2, 16, 128, 2048, [2048, 31], 2, torch.bfloat16),
+    ("plain decode, 4 rows", 8, 32, 8, 1, 128, 4096, [4096, 4000, 3000, 2000, 1000, 500, 65, 1], 2, torch.bfloat16),
+    ("head_dim 64, 40 rows", 2, 4, 2, 20, 64, 1024, [1000, 33], 1, torch.float16),
+    ("a tree of one and a half half-tiles", 1, 2, 2, 48, 128, 512, [512], 2, torch.bfloat16),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", KEY_HALVES_CASES, ids=lambda c: c[0])
+def test_key_halves_against_the_oracle(case):
+    """Units of at most 64 rows with two waves per 32-row block, each taking half of every tile's keys and
+    merging its state with its partner's before the epilogue. Against the oracle, against the 4-wave kernel
+    it stands in for, and with the merge inside the launch."""
+    name, bsz, hq, hkv, L, D, T, lens, splits, dtype = case
+    print("case:", name, flush=True)
+    x = make(81, bsz, hq, hkv, L, D, T, dtype, lens)
+    ref = oracle(x)
+    pc = prepare(x, _force_splits=splits, _force_kernel=_lib.KERNEL_MFMA_SPLIT_KEYS)
+    assert pc.plan.kernel == _lib.KERNEL_MFMA and pc.plan.rows_per_wg == 64 and pc.plan.mfma_loop == 2
+    out = pc.run().clone()
+    check(out, ref, dtype)
+    plain = prepare(x, _force_splits=splits, _force_kernel=_lib.KERNEL_MFMA)
+    assert plain.plan.rows_per_wg == 128 and plain.plan.mfma_loop == 0
+    torch.testing.assert_close(out.float(), plain.run().float(), **TOL[dtype])
+    if pc.plan.counter_elems:
+        check(pc.run_single_launch(), ref, dtype)
+
+
+@pytest.mark.gpu
+def test_key_halves_are_refused_where_they_do_not_exist():
+    x = make(82, 1, 8, 1, 16, 128, 256, torch.bfloat16, [256])                # 128-row units
+    with pytest.raises(ValueError, match="status -9"):
+        prepare(x, _force_kernel=_lib.KERNEL_MFMA_SPLIT_KEYS)
 
 
 # ---------------------------------------------------------------- head_dim 256: merge inside stage 1, paged caches
