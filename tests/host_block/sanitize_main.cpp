@@ -214,7 +214,7 @@ int main(int argc, char** argv) {
       {2, 2, 2, 3, 128, 160, 2, 16, {160, 17}, true, true},                // paged, packed mask
       {2, 8, 1, 20, 64, 192, 3, 0, {192, 70}, false, true, true},          // pipelined, merge inside the launch
       {1, 2, 2, 3, 256, 65, 1, 0, {65}, false, true},                      // head_dim 256, one key past a tile
-      {2, 4, 4, 26, 128, 200, 2, 0, {200, 33}, false, true, false, true},  // key halves: 26 rows, one key in the upper half of a tile
+      {2, 2, 2, 26, 128, 161, 2, 0, {161, 33}, false, true, false, true},  // key halves: 26 rows, one key in the upper half of a tile
       {2, 4, 1, 16, 64, 160, 2, 16, {160, 70}, true, true, true, true},    // key halves: 64 rows, paged, packed mask, merge inside the launch
   };
   const Case cases[] = {
