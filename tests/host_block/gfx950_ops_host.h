@@ -6,16 +6,26 @@
 // What is modelled: the data movement and arithmetic of each instruction - the 32x32x16 matrix
 // product with its operand and accumulator lane layout, the packed dot product, the half-wave swap,
 // the plain and the transposing LDS reads (addresses are offsets into the workgroup's LDS buffer), the
-// direct global->LDS load, ballots and barriers. What is NOT modelled: time. Every load has landed
-// when its statement ends, so the wait counters are no-ops and a wrong wait count cannot show here
-// (tests/test_kernel_asm.py and tests/test_wide_loop_model.py cover those). Matrix products accumulate
-// in fp32 in ascending k; the hardware's internal order may differ in the last bits.
+// direct global->LDS load, ballots and barriers. Matrix products accumulate in fp32 in ascending k; the
+// hardware's internal order may differ in the last bits.
+//
+// Time is modelled at its two extremes for the direct global->LDS loads, the only loads the kernel
+// waits for by count. By default a load lands the moment it is issued, the earliest it ever could:
+// a stage that is requested while another wave may still read it is then a data race for the thread
+// sanitizer. With FTA_HOST_LOADS_LAND_LATE set in the environment a load lands only when a vmcnt wait
+// of its wave forces it to (s_waitcnt vmcnt(N): all but the N youngest have landed; __syncthreads
+// waits for all), the latest the hardware allows: a wait that allows one load too many, or a missing
+// one, leaves NaN patterns in LDS for the products to find, reading a stage before the loading wave
+// has waited and passed a barrier is a data race, and a load still in flight when its thread leaves
+// the kernel aborts the run. (host_block_loads_land_late(int), exported by stage1_mfma_host.cpp, switches
+// the mode between launches.) LDS operand reads (lgkmcnt) are immediate in both modes.
 //
 // The hand-scheduled 64-row-wave loop (wide_loop_asm.inc) is assembly over fixed registers and does not
 // exist here: its macros abort.
 #pragma once
 #define FTA_GFX950_OPS_H
 #define FTA_WIDE_LOOP_ASM_INC
+#include <deque>
 #include <type_traits>
 
 #include "fta_device.h"
@@ -33,6 +43,33 @@ inline WaveExchange* exchange() { static WaveExchange x[16]; return x; }
 inline unsigned lane_id() { return threadIdx.x & 63; }
 inline WaveExchange& my_exchange() { return exchange()[threadIdx.x / 64]; }
 // Address of LDS byte `addr`, bounds-checked for an access of `bytes` bytes against what the launch asked for.
+// A direct global->LDS load of this lane that has not landed yet (late-landing mode).
+struct LoadInFlight {
+  const char* src;
+  uint32_t lds_addr;
+};
+inline bool& loads_land_late() { static bool late = std::getenv("FTA_HOST_LOADS_LAND_LATE") != nullptr; return late; }   // also host_block_loads_land_late()
+inline std::deque<LoadInFlight>& loads_in_flight() { static thread_local std::deque<LoadInFlight> q; return q; }
+inline char* lds_at(uint32_t addr, uint32_t bytes);
+// Lands the oldest loads of this lane until at most `allowed` are in flight (the counter retires in issue order).
+inline void land_all_but(size_t allowed) {
+  std::deque<LoadInFlight>& q = loads_in_flight();
+  while (q.size() > allowed) {
+    std::memcpy(lds_at(q.front().lds_addr, 16), q.front().src, 16);
+    q.pop_front();
+  }
+}
+inline void no_load_may_outlive_its_thread() {
+  if (!loads_in_flight().empty()) {
+    std::fprintf(stderr, "a thread left the kernel with %zu global->LDS loads in flight\n", loads_in_flight().size());
+    std::abort();
+  }
+}
+inline const bool hooks_installed = [] {
+  hooks().before_syncthreads = [] { land_all_but(0); };
+  hooks().at_thread_exit = no_load_may_outlive_its_thread;
+  return true;
+}();
 inline char* lds_at(uint32_t addr, uint32_t bytes) {
   if (static_cast<size_t>(addr) + bytes > lds_limit()) {
     std::fprintf(stderr, "LDS access of %u bytes at %u beyond the %zu bytes of this launch\n", bytes, addr, lds_limit());
@@ -112,7 +149,7 @@ inline float half_partner(float x, int /*lh*/) { return __shfl_xor(x, 32, 64); }
 inline float half_swap_max(float x, int lh) { return fmaxf(x, half_partner(x, lh)); }
 inline float half_swap_sum(float x, int lh) { return x + half_partner(x, lh); }
 
-template <int N> inline void wait_vmcnt() {}
+template <int N> inline void wait_vmcnt() { host_block::land_all_but(N); }
 template <int N> inline void wait_lgkm(u32x4&) {}
 template <int N> inline void wait_lgkm(u32x2&, u32x2&) {}
 inline void settle(f32x4&) {}
@@ -166,10 +203,16 @@ inline uint32_t lds_address(char* p) { return static_cast<uint32_t>(p - host_blo
 inline void host_load_block_to_lds(const char* lane_src, char* lds_block) {
   const uint32_t base = lds_address(lds_block);
   (void)uniform_ptr(lds_block);
-  std::memcpy(host_block::lds_at(base + 16 * host_block::lane_id(), 16), lane_src, 16);
+  const uint32_t mine = base + 16 * host_block::lane_id();
+  if (host_block::loads_land_late()) {
+    (void)host_block::lds_at(mine, 16);                        // the bounds check, at issue
+    host_block::loads_in_flight().push_back({lane_src, mine});
+  } else {
+    std::memcpy(host_block::lds_at(mine, 16), lane_src, 16);
+  }
 }
 #define FTA_LOAD_BLOCK_TO_LDS(lane_src, lds_block) host_load_block_to_lds(lane_src, lds_block)
-inline void workgroup_barrier() { __syncthreads(); }
+inline void workgroup_barrier() { host_block::current()->all.arrive_and_wait(); }   // s_barrier alone: no wait for memory operations
 inline void schedule_fence() {}
 inline bool wave_any(bool pred) {
   int any = pred ? 1 : 0;

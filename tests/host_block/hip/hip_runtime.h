@@ -58,7 +58,20 @@ inline size_t& lds_limit() { static size_t bytes = 0; return bytes; }   // dynam
 inline thread_local dim3 threadIdx, blockIdx;
 inline dim3 blockDim, gridDim;
 
-inline void __syncthreads() { host_block::current()->all.arrive_and_wait(); }
+namespace host_block {
+// Hooks of a stand-in that keeps per-thread state of its own (gfx950_ops_host.h: loads in flight): called by every
+// thread before __syncthreads (which waits for all of a thread's memory operations on the GPU) and when a thread
+// leaves the kernel.
+struct Hooks {
+  void (*before_syncthreads)() = nullptr;
+  void (*at_thread_exit)() = nullptr;
+};
+inline Hooks& hooks() { static Hooks h; return h; }
+}  // namespace host_block
+inline void __syncthreads() {
+  if (host_block::hooks().before_syncthreads) host_block::hooks().before_syncthreads();
+  host_block::current()->all.arrive_and_wait();
+}
 inline void host_wave_barrier() { host_block::current()->wave[threadIdx.x / 64]->arrive_and_wait(); }
 
 template <typename T>
@@ -112,6 +125,7 @@ inline hipError_t launch(Kernel kern, dim3 grid, dim3 block, const Params& param
         threadIdx = dim3(t);
         blockIdx = dim3(id);
         kern(params);
+        if (hooks().at_thread_exit) hooks().at_thread_exit();
         state.all.arrive_and_drop();
         state.wave[t / 64]->arrive_and_drop();
       });

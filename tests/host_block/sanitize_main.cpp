@@ -11,6 +11,8 @@
 
 #include "fta.h"
 
+extern "C" void host_block_loads_land_late(int late) __attribute__((weak));   // only in builds with the MFMA kernel
+
 namespace {
 struct Case {
   int bsz, hq, hkv, L, D, tmax, splits, page;   // page 0 = contiguous caches
@@ -206,8 +208,11 @@ int run_append() {
 }  // namespace
 
 int main(int argc, char** argv) {
-  // "mfma" as first argument: the build holds the MFMA kernel (stage1_mfma_host.cpp), run its cases as well
+  // "mfma" as first argument: the build holds the MFMA kernel (stage1_mfma_host.cpp), run its cases as well;
+  // "both" as second: run them once with global->LDS loads that land when issued and once with loads that land
+  // only when a wait forces them to (a stage read before its loader has waited and passed a barrier is then a race)
   const bool with_mfma = argc > 1 && std::strcmp(argv[1], "mfma") == 0;
+  const bool both = with_mfma && argc > 2 && std::strcmp(argv[2], "both") == 0;
   const Case mfma_cases[] = {
       {2, 4, 2, 5, 64, 200, 2, 0, {200, 77}, false, true},                 // 4 waves, rings of 2; ragged last tiles
       {1, 8, 1, 20, 128, 390, 1, 0, {390}, false, true},                   // 8 waves pipelined through rings of 3 and 5, ragged end
@@ -228,7 +233,11 @@ int main(int argc, char** argv) {
   int bad = 0;
   for (const Case& c : cases) bad += run(c);
   if (with_mfma)
-    for (const Case& c : mfma_cases) bad += run(c);
+    for (int late = 0; late <= (both ? 1 : 0); ++late) {
+      if (host_block_loads_land_late) host_block_loads_land_late(late);
+      std::printf("global->LDS loads land %s\n", late ? "late" : "when issued");
+      for (const Case& c : mfma_cases) bad += run(c);
+    }
   bad += run_append();
   std::printf(bad ? "FAILED\n" : "clean\n");
   return bad;

@@ -11,3 +11,7 @@
 namespace fta {
 int launch_stage1_mfma_wide(const KernelParams&, int, int, void*) { return FTA_ERR_UNSUPPORTED; }
 }  // namespace fta
+
+// Switches the model of the direct global->LDS loads between launches: 0 = they land when issued, 1 = they land
+// when a wait of their wave forces them to (gfx950_ops_host.h).
+extern "C" void host_block_loads_land_late(int late) { host_block::loads_land_late() = late != 0; }

@@ -11,8 +11,9 @@ on the host (tests/test_wide_loop_model.py executes that one).
 What this pins without a GPU: the work decomposition and addressing of the kernel (units, row blocks, splits,
 chunk by the batch's longest sequence, strides, paged lookups, ragged and tree tiles, the ring slots), its
 lane layouts, the online softmax with the deferred rescale, the compensated masked tiles, the epilogue, and
-the merge inside the launch with counters. What it cannot show: anything about time (loads land at once here,
-so wait counts are not exercised), and the last bits of the hardware's accumulation order.
+the merge inside the launch with counters. Time is modelled at its extremes only: global->LDS loads land when
+issued, or (test_hand_counted_waits_...) as late as the kernel's vmcnt waits allow. Not shown: LDS operand reads
+in flight (lgkmcnt; tests/test_kernel_asm.py pins those) and the last bits of the hardware's accumulation order.
 
 TEST INFRASTRUCTURE ONLY: nothing under flash_tree_attn_amd/ knows of this build."""
 import ctypes as C
@@ -55,8 +56,16 @@ def host_lib(tmp_path_factory):
     for name in ("fta_decode", "fta_decode_stage1", "fta_decode_stage2"):
         getattr(lib, name).argtypes = [C.POINTER(_lib.FtaArgs), C.c_void_p]
     lib.fta_plan.argtypes = [C.POINTER(_lib.FtaArgs), C.c_int, C.POINTER(_lib.FtaPlanOut)]
+    lib.host_block_loads_land_late.argtypes = [C.c_int]
     assert lib.fta_abi_version() == _lib.ABI_VERSION
     return lib
+
+
+@pytest.fixture(autouse=True)
+def loads_land_when_issued(host_lib):
+    host_lib.host_block_loads_land_late(0)
+    yield
+    host_lib.host_block_loads_land_late(0)
 
 
 def clamped(x, lens, tmax):
@@ -245,3 +254,37 @@ def test_key_halves_are_refused_where_they_do_not_exist(host_lib):
         x = make(1, 1, hq, 1, L, D, 64, torch.float16, [64])
         with pytest.raises(AssertionError):
             HostCall(host_lib, x, kernel=SPLIT_KEYS)
+
+
+@pytest.mark.parametrize("shape", [
+    # bsz hq hkv L  D    tmax dtype           lens         splits kernel      rows_per_wg
+    (2, 4, 2, 5, 64, 300, torch.bfloat16, [200, 77], 2, MFMA, 128),              # rings of 2
+    (1, 8, 1, 20, 128, 512, torch.float16, [470], 1, MFMA, 256),                 # the 8-wave pipeline: K ring 3, V ring 5, waits of 1 .. 4 tiles
+    (1, 8, 1, 20, 128, 256, torch.bfloat16, [70], 1, MFMA, 256),                 # the same with fewer tiles than its rings hold
+    (1, 2, 2, 3, 256, 256, torch.float16, [100], 1, MFMA, 128),                  # head_dim 256: 16 loads per wave and tile
+    (2, 4, 4, 26, 128, 320, torch.float16, [300, 64], 3, SPLIT_KEYS, 64),        # key halves
+])
+def test_hand_counted_waits_hold_when_loads_land_as_late_as_they_may(host_lib, shape):
+    """The kernel waits for its tile loads by count (s_waitcnt vmcnt(N) with N from the ring's state). Here a
+    load lands only when such a wait, or __syncthreads, forces it to: a count that allows one load too many
+    leaves NaN patterns where the products read. (Checked by hand: with the wait for "one younger tile" allowing
+    two, this fails and the default mode does not.)"""
+    bsz, hq, hkv, L, D, tmax, dtype, lens, splits, kernel, rows_per_wg = shape
+    x = make(31, bsz, hq, hkv, L, D, tmax, dtype, lens)
+    call = HostCall(host_lib, x, splits=splits, kernel=kernel)
+    assert call.plan.rows_per_wg == rows_per_wg
+    host_lib.host_block_loads_land_late(1)
+    out = call.run()
+    torch.testing.assert_close(out.float(), oracle(x), **TOL[dtype])
+    paged_ok = D != 256
+    if paged_ok:      # paged: the table lookups sit between the requests and the waits
+        page, per_seq = 64, tmax // 64
+        perm = torch.randperm(bsz * per_seq, generator=torch.Generator().manual_seed(5)).view(bsz, per_seq)
+        kp = torch.empty((bsz * per_seq, hkv, page, D), dtype=dtype)
+        vp = torch.empty_like(kp)
+        for b in range(bsz):
+            for pg in range(per_seq):
+                kp[perm[b, pg]] = x["k_cache"][b, :, pg * page:(pg + 1) * page]
+                vp[perm[b, pg]] = x["v_cache"][b, :, pg * page:(pg + 1) * page]
+        paged = HostCall(host_lib, x, splits=splits, hint=tmax, tables=perm.to(torch.int32).contiguous(), pools=(kp, vp), kernel=kernel)
+        torch.testing.assert_close(paged.run().float(), oracle(x), **TOL[dtype])
