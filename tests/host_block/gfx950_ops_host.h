@@ -18,7 +18,8 @@
 // one, leaves NaN patterns in LDS for the products to find, reading a stage before the loading wave
 // has waited and passed a barrier is a data race, and a load still in flight when its thread leaves
 // the kernel aborts the run. (host_block_loads_land_late(int), exported by stage1_mfma_host.cpp, switches
-// the mode between launches.) LDS operand reads (lgkmcnt) are immediate in both modes.
+// the mode between launches.) LDS operand reads are in flight until their lgkmcnt wait in both modes (see
+// wait_lgkm below).
 //
 // The hand-scheduled 64-row-wave loop (wide_loop_asm.inc) is assembly over fixed registers and does not
 // exist here: its macros abort.
@@ -59,9 +60,18 @@ inline void land_all_but(size_t allowed) {
     q.pop_front();
   }
 }
+// An LDS operand read of this lane whose data no lgkmcnt wait has handed to a register yet.
+struct LdsReadInFlight {
+  unsigned char data[16];
+};
+inline std::deque<LdsReadInFlight>& lds_reads_in_flight() { static thread_local std::deque<LdsReadInFlight> q; return q; }
 inline void no_load_may_outlive_its_thread() {
   if (!loads_in_flight().empty()) {
     std::fprintf(stderr, "a thread left the kernel with %zu global->LDS loads in flight\n", loads_in_flight().size());
+    std::abort();
+  }
+  if (!lds_reads_in_flight().empty()) {
+    std::fprintf(stderr, "a thread left the kernel with %zu LDS operand reads that no wait has landed\n", lds_reads_in_flight().size());
     std::abort();
   }
 }
@@ -150,15 +160,48 @@ inline float half_swap_max(float x, int lh) { return fmaxf(x, half_partner(x, lh
 inline float half_swap_sum(float x, int lh) { return x + half_partner(x, lh); }
 
 template <int N> inline void wait_vmcnt() { host_block::land_all_but(N); }
-template <int N> inline void wait_lgkm(u32x4&) {}
-template <int N> inline void wait_lgkm(u32x2&, u32x2&) {}
+// LDS operand reads are asynchronous too: the destination registers hold nothing until an
+// s_waitcnt lgkmcnt(N) has let all but the N youngest reads land (LDS returns data in issue order).
+// The kernel issues such reads ahead of their use and names, at each wait, the registers that the
+// wait makes valid. Here a read returns a NaN pattern and queues its data; a wait hands the data of
+// the reads it lands to the registers it names, and insists that these are exactly the reads it lands:
+// a count that is one too high leaves the pattern in place (and aborts), one too low lands a read that
+// no register is named for (and aborts).
+namespace lds_reads {
+inline std::deque<host_block::LdsReadInFlight>& queue() { return host_block::lds_reads_in_flight(); }
+template <typename V> inline V issue(const void* data) {
+  host_block::LdsReadInFlight r;
+  std::memcpy(r.data, data, sizeof(V));
+  queue().push_back(r);
+  V poison;
+  std::memset(&poison, 0xFF, sizeof(V));
+  return poison;
+}
+template <typename V> inline void land_into(V& reg) {
+  std::memcpy(&reg, queue().front().data, sizeof(V));
+  queue().pop_front();
+}
+inline void expect_landing(size_t allowed_in_flight, size_t named) {
+  if (queue().size() != allowed_in_flight + named) {
+    std::fprintf(stderr, "s_waitcnt lgkmcnt(%zu) with %zu LDS reads in flight names %zu register group(s)\n", allowed_in_flight, queue().size(), named);
+    std::abort();
+  }
+}
+}  // namespace lds_reads
+template <int N> inline void wait_lgkm(u32x4& a) {
+  lds_reads::expect_landing(N, 1);
+  lds_reads::land_into(a);
+}
+template <int N> inline void wait_lgkm(u32x2& a, u32x2& b) {
+  lds_reads::expect_landing(N, 2);
+  lds_reads::land_into(a);
+  lds_reads::land_into(b);
+}
 inline void settle(f32x4&) {}
 
 template <int OFF>
 inline u32x4 lds_read_b128(uint32_t addr) {
-  u32x4 v;
-  std::memcpy(&v, host_block::lds_at(addr + OFF, 16), 16);
-  return v;
+  return lds_reads::issue<u32x4>(host_block::lds_at(addr + OFF, 16));
 }
 // ds_read_b64_tr_b16: the 16 lanes of a group each fetch 8 bytes (four 16-bit values). The 64 values of
 // the group, read as four rows of sixteen (row e = the values of lanes 4e .. 4e+3 in order), come back
@@ -175,9 +218,7 @@ inline u32x2 lds_read_tr16_b64(uint32_t addr) {
     std::memcpy(&out[e], x.bytes[src] + 2 * (s % 4), 2);
   }
   host_wave_barrier();
-  u32x2 v;
-  std::memcpy(&v, out, 8);
-  return v;
+  return lds_reads::issue<u32x2>(out);
 }
 
 inline void store_b128_device(void* ptr, f32x4 v) { std::memcpy(ptr, &v, 16); }

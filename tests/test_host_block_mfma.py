@@ -12,8 +12,9 @@ What this pins without a GPU: the work decomposition and addressing of the kerne
 chunk by the batch's longest sequence, strides, paged lookups, ragged and tree tiles, the ring slots), its
 lane layouts, the online softmax with the deferred rescale, the compensated masked tiles, the epilogue, and
 the merge inside the launch with counters. Time is modelled at its extremes only: global->LDS loads land when
-issued, or (test_hand_counted_waits_...) as late as the kernel's vmcnt waits allow. Not shown: LDS operand reads
-in flight (lgkmcnt; tests/test_kernel_asm.py pins those) and the last bits of the hardware's accumulation order.
+issued, or (test_hand_counted_waits_...) as late as the kernel's vmcnt waits allow; LDS operand reads stay in
+flight until the lgkmcnt wait that names their registers, and every such wait must land exactly the reads it
+names (the stand-in aborts otherwise). Not shown: the last bits of the hardware's accumulation order, and speed.
 
 TEST INFRASTRUCTURE ONLY: nothing under flash_tree_attn_amd/ knows of this build."""
 import ctypes as C
