@@ -13,8 +13,8 @@
 // waits for by count. By default a load lands the moment it is issued, the earliest it ever could:
 // a stage that is requested while another wave may still read it is then a data race for the thread
 // sanitizer. With FTA_HOST_LOADS_LAND_LATE set in the environment a load lands only when a vmcnt wait
-// of its wave forces it to (s_waitcnt vmcnt(N): all but the N youngest have landed; __syncthreads
-// waits for all), the latest the hardware allows: a wait that allows one load too many, or a missing
+// of its wave forces it to (s_waitcnt vmcnt(N): all but the N youngest have landed; nothing else
+// counts, not even __syncthreads, whose own wait the kernel does not rely on), the latest the hardware allows: a wait that allows one load too many, or a missing
 // one, leaves NaN patterns in LDS for the products to find, reading a stage before the loading wave
 // has waited and passed a barrier is a data race, and a load still in flight when its thread leaves
 // the kernel aborts the run. (host_block_loads_land_late(int), exported by stage1_mfma_host.cpp, switches
@@ -76,7 +76,6 @@ inline void no_load_may_outlive_its_thread() {
   }
 }
 inline const bool hooks_installed = [] {
-  hooks().before_syncthreads = [] { land_all_but(0); };
   hooks().at_thread_exit = no_load_may_outlive_its_thread;
   return true;
 }();

@@ -59,19 +59,14 @@ inline thread_local dim3 threadIdx, blockIdx;
 inline dim3 blockDim, gridDim;
 
 namespace host_block {
-// Hooks of a stand-in that keeps per-thread state of its own (gfx950_ops_host.h: loads in flight): called by every
-// thread before __syncthreads (which waits for all of a thread's memory operations on the GPU) and when a thread
-// leaves the kernel.
+// Hook of a stand-in that keeps per-thread state of its own (gfx950_ops_host.h: loads in flight): called by every
+// thread when it leaves the kernel.
 struct Hooks {
-  void (*before_syncthreads)() = nullptr;
   void (*at_thread_exit)() = nullptr;
 };
 inline Hooks& hooks() { static Hooks h; return h; }
 }  // namespace host_block
-inline void __syncthreads() {
-  if (host_block::hooks().before_syncthreads) host_block::hooks().before_syncthreads();
-  host_block::current()->all.arrive_and_wait();
-}
+inline void __syncthreads() { host_block::current()->all.arrive_and_wait(); }
 inline void host_wave_barrier() { host_block::current()->wave[threadIdx.x / 64]->arrive_and_wait(); }
 
 template <typename T>

@@ -267,7 +267,7 @@ def test_key_halves_are_refused_where_they_do_not_exist(host_lib):
 ])
 def test_hand_counted_waits_hold_when_loads_land_as_late_as_they_may(host_lib, shape):
     """The kernel waits for its tile loads by count (s_waitcnt vmcnt(N) with N from the ring's state). Here a
-    load lands only when such a wait, or __syncthreads, forces it to: a count that allows one load too many
+    load lands only when such a wait forces it to (not even __syncthreads counts): a count that allows one load too many
     leaves NaN patterns where the products read. (Checked by hand: with the wait for "one younger tile" allowing
     two, this fails and the default mode does not.)"""
     bsz, hq, hkv, L, D, tmax, dtype, lens, splits, kernel, rows_per_wg = shape
