@@ -21,8 +21,8 @@
 // the mode between launches.) LDS operand reads are in flight until their lgkmcnt wait in both modes (see
 // wait_lgkm below).
 //
-// The hand-scheduled 64-row-wave loop (wide_loop_asm.inc) is assembly over fixed registers and does not
-// exist here: its macros abort.
+// The hand-scheduled 64-row-wave loop (wide_loop_asm.inc) is assembly over fixed registers: its macros
+// abort here, unless the build supplies them as calls of the interpreter in gfx950_asm_host.h.
 #pragma once
 #define FTA_GFX950_OPS_H
 #define FTA_WIDE_LOOP_ASM_INC
@@ -90,6 +90,10 @@ inline char* lds_at(uint32_t addr, uint32_t bytes) {
 
 #define FTA_WAVES_PER_EU(n)
 #define __HIP_MEMORY_SCOPE_AGENT 4
+// The assembly statements of the 64-row-wave loop: absent (a kernel that reaches one aborts), unless the build
+// names a rendering of them as interpreter calls (FTA_HOST_WIDE_LOOP_INC, made from the same generator output as
+// wide_loop_asm.inc by tests/test_host_block_wide.py; included at the end of this file).
+#ifndef FTA_HOST_WIDE_LOOP_INC
 #define FTA_WIDE_LOOP_128_BF16() host_block::no_assembly()
 #define FTA_WIDE_LOOP_128_F16() host_block::no_assembly()
 #define FTA_WIDE_LOOP_64_BF16() host_block::no_assembly()
@@ -102,6 +106,7 @@ inline char* lds_at(uint32_t addr, uint32_t bytes) {
 #define FTA_WIDE_MASKED_64_BF16_H1() host_block::no_assembly()
 #define FTA_WIDE_MASKED_64_F16_H0() host_block::no_assembly()
 #define FTA_WIDE_MASKED_64_F16_H1() host_block::no_assembly()
+#endif
 
 namespace fta {
 namespace {
@@ -262,3 +267,8 @@ inline bool wave_any(bool pred) {
 
 }  // namespace
 }  // namespace fta
+
+#ifdef FTA_HOST_WIDE_LOOP_INC
+#include "gfx950_asm_host.h"
+#include FTA_HOST_WIDE_LOOP_INC
+#endif

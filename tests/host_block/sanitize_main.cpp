@@ -21,6 +21,7 @@ struct Case {
   bool mfma = false;    // bf16 tensors through the MFMA kernel (where the build has it) instead of fp32 through the shuffle kernel
   bool fused = false;   // with counters: the merge inside stage 1's launch
   bool key_halves = false;   // the MFMA kernel's form for small units: two waves per 32-row block
+  bool wide = false;         // the MFMA kernel's 64-row-wave form, its assembly statements interpreted
 };
 
 std::mt19937 rng(1234);
@@ -109,7 +110,7 @@ int run(const Case& c) {
   a.mask_kind = c.packed ? FTA_MASK_PACKED_U64 : FTA_MASK_ADDITIVE_F32;
   a.bsz = c.bsz; a.num_q_heads = c.hq; a.num_kv_heads = c.hkv; a.cur_heads = c.hkv; a.q_len = c.L; a.head_dim = c.D;
   a.block_size = 64; a.dtype = c.mfma ? FTA_BF16 : FTA_F32; a.len_dtype = FTA_I64; a.force_splits = c.splits;
-  a.force_kernel = c.key_halves ? FTA_KERNEL_MFMA_SPLIT_KEYS : c.mfma ? FTA_KERNEL_MFMA : FTA_KERNEL_SHUFFLE;
+  a.force_kernel = c.wide ? FTA_KERNEL_MFMA_WIDE : c.key_halves ? FTA_KERNEL_MFMA_SPLIT_KEYS : c.mfma ? FTA_KERNEL_MFMA : FTA_KERNEL_SHUFFLE;
   a.sm_scale = 1.f / std::sqrt((float)c.D);
   const long long LD = (long long)c.L * c.D;
   a.q_stride[0] = c.hq * LD; a.q_stride[1] = LD; a.q_stride[2] = c.D;
@@ -221,6 +222,8 @@ int main(int argc, char** argv) {
       {1, 2, 2, 3, 256, 65, 1, 0, {65}, false, true},                      // head_dim 256, one key past a tile
       {2, 2, 2, 26, 128, 161, 2, 0, {161, 33}, false, true, false, true},  // key halves: 26 rows, one key in the upper half of a tile
       {2, 4, 1, 16, 64, 160, 2, 16, {160, 70}, true, true, true, true},    // key halves: 64 rows, paged, packed mask, merge inside the launch
+      {1, 4, 1, 64, 128, 300, 1, 0, {300}, false, true, false, false, true},           // 64-row waves: tree tile, 4 tiles in the loop, ragged tail
+      {2, 8, 1, 32, 64, 200, 2, 0, {200, 64}, true, true, true, false, true},          // 64-row waves: head_dim 64, packed mask, merge inside the launch
   };
   const Case cases[] = {
       {2, 4, 2, 5, 32, 100, 2, 0, {100, 37}, false},          // ragged tiles at the end of cache and tree

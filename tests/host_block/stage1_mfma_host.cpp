@@ -8,9 +8,11 @@
 #include "stage1_mfma.hip"
 #include "stage1_mfma_splitkeys.hip"
 
+#ifndef FTA_HOST_WITH_WIDE_UNIT   // defined when stage1_mfma_wide_host.cpp is part of the build
 namespace fta {
 int launch_stage1_mfma_wide(const KernelParams&, int, int, void*) { return FTA_ERR_UNSUPPORTED; }
 }  // namespace fta
+#endif
 
 // Switches the model of the direct global->LDS loads between launches: 0 = they land when issued, 1 = they land
 // when a wait of their wave forces them to (gfx950_ops_host.h).

@@ -5,8 +5,8 @@ the instruction wrappers of csrc/gfx950_ops.h replaced by arithmetic stand-ins (
 32x32x16 matrix product in its lane layout, the transposing LDS read, the direct global->LDS load with
 bounds-checked LDS addresses, ...), one host thread per GPU thread, and runs it through the library's own C
 entry points. All three compiled loop variants run: 4 waves x 32 rows with rings of 2 (also head_dim 256),
-and 8 waves x 32 rows software-pipelined over whole tiles. The assembly loop of 64-row waves does not exist
-on the host (tests/test_wide_loop_model.py executes that one).
+and 8 waves x 32 rows software-pipelined over whole tiles. (The 64-row-wave kernel, whose loop is assembly, runs
+in tests/test_host_block_wide.py with its statements interpreted.)
 
 What this pins without a GPU: the work decomposition and addressing of the kernel (units, row blocks, splits,
 chunk by the batch's longest sequence, strides, paged lookups, ragged and tree tiles, the ring slots), its
