@@ -18,6 +18,7 @@ double-precision attention.
     without the barrier of the MFMA kernel's synchronisation point 192.)"""
 import os
 import subprocess
+from concurrent.futures import ThreadPoolExecutor
 
 import pytest
 
@@ -28,18 +29,27 @@ CLANG = os.path.join(os.path.dirname(fta_build.HIPCC), "..", "llvm", "bin", "cla
 SOURCES = ["fta_host.cpp", "stage1_shuffle.hip", "stage2_merge.hip", "append_kv.hip"]
 
 
-@pytest.mark.parametrize("sanitize", ["address,undefined", "thread"])
-def test_host_build_is_clean_under(sanitize, tmp_path):
+def test_host_build_is_clean_under_the_sanitizers(tmp_path):
     if not os.path.exists(CLANG):
         pytest.skip("no host clang++")
     from test_host_block_wide import build_host_library_with_wide
-    exe = build_host_library_with_wide(str(tmp_path), extra_flags=["-g", f"-fsanitize={sanitize}", "-fno-omit-frame-pointer"], link_flags=[f"-fsanitize={sanitize}"],
-                                       extra_sources=[os.path.join(HERE, "host_block", "sanitize_main.cpp")], output="sanitize_host", shared=False)
+    kinds = ["address,undefined", "thread"]
+
+    def build(sanitize):
+        out = tmp_path / sanitize.split(",")[0]
+        out.mkdir()
+        return build_host_library_with_wide(str(out), extra_flags=["-g", f"-fsanitize={sanitize}", "-fno-omit-frame-pointer"], link_flags=[f"-fsanitize={sanitize}"],
+                                            extra_sources=[os.path.join(HERE, "host_block", "sanitize_main.cpp")], output="sanitize_host", shared=False)
+
+    with ThreadPoolExecutor(max_workers=2) as pool:      # both builds, then both runs, side by side
+        exes = list(pool.map(build, kinds))
     env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0", UBSAN_OPTIONS="halt_on_error=1", TSAN_OPTIONS="halt_on_error=0")
     # under the thread sanitizer the MFMA cases run twice: loads that land when issued, then loads that land as late as the waits allow
-    r = subprocess.run([exe, "mfma"] + (["both"] if sanitize == "thread" else []), capture_output=True, text=True, timeout=900, env=env)
-    text = r.stdout + r.stderr
-    for sign in ("AddressSanitizer", "runtime error", "data race", "ThreadSanitizer", "FAILED"):
-        assert sign not in text, text[-3000:]
-    assert r.returncode == 0 and text.strip().endswith("clean"), text[-2000:]
-    assert text.count("bf16/mfma") == (18 if sanitize == "thread" else 9), text[-2000:]
+    runs = [subprocess.Popen([exe, "mfma"] + (["both"] if sanitize == "thread" else []), stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env)
+            for exe, sanitize in zip(exes, kinds)]
+    for run, sanitize in zip(runs, kinds):
+        text = run.communicate(timeout=900)[0]
+        for sign in ("AddressSanitizer", "runtime error", "data race", "ThreadSanitizer", "FAILED"):
+            assert sign not in text, (sanitize, text[-3000:])
+        assert run.returncode == 0 and text.strip().endswith("clean"), (sanitize, text[-2000:])
+        assert text.count("bf16/mfma") == (18 if sanitize == "thread" else 9), (sanitize, text[-2000:])

@@ -142,8 +142,8 @@ def test_64_row_wave_kernel_on_host_threads(host_lib, case):
 
 
 def test_64_row_wave_kernel_partials_and_merge_inside_the_launch(host_lib):
-    lens, tmax, S = [330, 130, 0], 2048, 3
-    x = make(77, 3, 4, 1, 64, 128, tmax, torch.bfloat16, lens)
+    lens, tmax, S = [330, 0], 2048, 3
+    x = make(77, 2, 3, 1, 64, 128, tmax, torch.bfloat16, lens)
     call = HostCall(host_lib, x, splits=S, kernel=WIDE)
     chunk = call.plan.chunk_for(max(lens))
     assert call.plan.num_splits == S and chunk < call.plan.chunk
