@@ -824,10 +824,12 @@ stage1_mfma_kernel(const KernelParams p) {
   // for the tree block). key0 is the first key of the half. The additive terms are gathered
   // here; the step itself is assembly with the register map of the loop (gen_wide_loop.py:
   // gen_masked), so that O, Q, m and l stay where the loop wants them.
-  auto masked_half = [&](auto h_c, auto tree_c, int t, int key0, int key_lim) __attribute__((always_inline)) {
-    constexpr int H = decltype(h_c)::value;
+  // The additive terms of one half: [qb][16] in the accumulator layout, mask * log2(e), -inf past the key
+  // limit. For the tree block these are global loads; phase A issues them ahead of the synchronisation point
+  // of their tile, so that they are in flight while the wave waits for the tile and the barrier (the
+  // statement takes them as register inputs: gathered right in front of it, their whole latency would show).
+  auto gather_madd = [&](auto tree_c, int key0, int key_lim, float (&w_madd)[32]) __attribute__((always_inline)) {
     constexpr bool TREE = decltype(tree_c)::value;
-    float w_madd[32];   // [qb][16], in the accumulator layout: mask * log2(e), -inf past the key limit
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
       float mv[16];
@@ -863,6 +865,9 @@ stage1_mfma_kernel(const KernelParams p) {
         w_madd[qb * 16 + r] = j < key_lim ? add : neg_inf();
       }
     }
+  };
+  auto masked_half = [&](auto h_c, int t, const float (&w_madd)[32]) __attribute__((always_inline)) {
+    constexpr int H = decltype(h_c)::value;
     float w_o[32 * DB], w_m[2] = {m_run[0], m_run[1]}, w_l[2] = {l_run[0], l_run[1]};
     uint32_t w_q[8 * KS];
 #pragma unroll
@@ -967,10 +972,17 @@ stage1_mfma_kernel(const KernelParams p) {
     constexpr std::integral_constant<int, 1> h1{};
     // phase A: the tree tiles, half by half, each half a complete masked step
     for (int u = 0; u < tree_tiles; ++u) {
+      // (only the first half's terms go ahead: the second half's would have to live through the first statement,
+      // which leaves the compiler too few registers to hold them; their cache lines are warm by then)
+      float madd[32];
+      if (wave_active) gather_madd(std::true_type{}, u * kKeyTile, L, madd);
       sync_point(u, u, u, ntiles);
       if (!wave_active) continue;
-      masked_half(h0, std::true_type{}, u, u * kKeyTile, L);
-      if (u * kKeyTile + 32 < L) masked_half(h1, std::true_type{}, u, u * kKeyTile + 32, L);
+      masked_half(h0, u, madd);
+      if (u * kKeyTile + 32 < L) {
+        gather_madd(std::true_type{}, u * kKeyTile + 32, L, madd);
+        masked_half(h1, u, madd);
+      }
     }
     // phase B: the full cache tiles through the half-tile pipeline. One synchronisation
     // point per tile, between its two steps: by then every wave has read all of K of tile
@@ -1045,8 +1057,13 @@ stage1_mfma_kernel(const KernelParams p) {
       sync_point(t, t, t, ntiles);
       if (wave_active) {
         const int key0 = kv_start + (t - c0) * kKeyTile;
-        masked_half(h0, std::false_type{}, t, key0, kv_end);
-        if (key0 + 32 < kv_end) masked_half(h1, std::false_type{}, t, key0 + 32, kv_end);
+        float madd[32];
+        gather_madd(std::false_type{}, key0, kv_end, madd);
+        masked_half(h0, t, madd);
+        if (key0 + 32 < kv_end) {
+          gather_madd(std::false_type{}, key0 + 32, kv_end, madd);
+          masked_half(h1, t, madd);
+        }
       }
     }
     wait_vmcnt<0>();   // tiles requested past the end are still landing: they must not outlive the workgroup's LDS
