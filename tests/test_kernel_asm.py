@@ -256,3 +256,30 @@ def test_generator_rejects_issue_hazards():
     end = max(i for i, l in enumerate(body) if l.startswith("s_nop 15"))
     with pytest.raises(AssertionError, match="statement ends"):
         gen.hazards(body[:end] + ["s_nop 3"] + body[end + 1:], "fence")
+
+
+def test_instruction_mix_of_the_generated_loop_per_tile():
+    """What one wave issues per 64-key tile in the steady state of the 64-row-wave loop (the text between the loop
+    label and the backward branch; the exact redo sits outside of it). These are the figures the design argues with:
+    every K or V fragment read feeds two matrix products, 3.4 vector instructions per product, one barrier and one
+    round of tile requests per tile. A change of the generator that moves them has to move this test."""
+    import collections
+    gen = _generator()
+    for D, want in ((128, dict(mfma=64, lds=48, dma=8)), (64, dict(mfma=32, lds=24, dma=4))):
+        for dtype in ("bf16", "f16"):
+            body = gen.gen(D, dtype)
+            first = next(i for i, l in enumerate(body) if l.startswith(".Lloop_"))
+            last = next(i for i, l in enumerate(body) if l.startswith("s_cbranch_scc1 .Lloop_"))
+            mix = collections.Counter()
+            for line in body[first + 1:last + 1]:
+                line = line.split(";")[0].strip()
+                if not line or line.endswith(":"):
+                    continue
+                op = line.split()[0]
+                kind = ("mfma" if op.startswith("v_mfma") else "lds" if op.startswith("ds_") else "dma" if op.startswith("global_load_lds") else
+                        "exp" if op.startswith("v_exp") else "valu" if op.startswith("v_") else "barrier" if op == "s_barrier" else "other")
+                mix[kind] += 1
+            assert {k: mix[k] for k in want} == want, (D, dtype, mix)
+            assert mix["lds"] * 4 == mix["mfma"] * 3                       # 2 K + 1 V^T pair of reads per four products
+            assert mix["exp"] == 64 and mix["barrier"] == 1               # 64 rows x 64 keys over 64 lanes; one synchronisation point
+            assert mix["valu"] + mix["exp"] <= 216, (D, dtype, mix)        # 3.4 per matrix product at head_dim 128
