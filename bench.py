@@ -53,6 +53,9 @@ def parse():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run plain device copies of a known size (reference point for rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
+    ap.add_argument("--compare", default="", metavar="K1,K2,...",
+                    help="only time the call with each of these stage-1 kernels (names as for --kernel) on the same inputs, in one "
+                         "process and one warm card, and print the medians side by side as one JSON line")
     return ap.parse_args()
 
 
@@ -208,6 +211,57 @@ def bench_append(args, cfg, dev):
     }))
 
 
+def compare_kernels(args, cfg, x, mask_arg, names, kernel_ids):
+    """Times the whole call and stage 1 alone with each named stage-1 kernel on the same contiguous inputs: one settle
+    phase, then per kernel a warm-up and event-timed batches of 25 calls, kernels taking turns batch by batch so that a
+    drift of the card's clocks hits all of them alike. Each kernel's result is checked against the first one's."""
+    import torch
+    from flash_tree_attn_amd import prepare
+    from flash_tree_attn_amd.synthetic import algorithmic_bytes
+    for n in names:
+        if n not in kernel_ids:
+            raise SystemExit(f"--compare: no kernel named {n!r}")
+    kv_sets = len(x["k_caches"])
+    calls = {n: [prepare(x["q"], kc, vc, x["current_k"], x["current_v"], mask_arg, x["kv_seq_len"], cfg.block_size, None, None, None, None,
+                         x["sm_scale"], cfg.kv_group_num, _force_splits=args.splits, _force_kernel=kernel_ids[n])
+                 for kc, vc in zip(x["k_caches"], x["v_caches"])] for n in names}
+    tol = dict(atol=2e-3, rtol=1e-2) if cfg.dtype != torch.float32 else dict(atol=2e-5, rtol=1e-4)
+    first = calls[names[0]][0].run().float().clone()
+    for n in names[1:]:
+        torch.testing.assert_close(calls[n][0].run().float(), first, **tol)
+    stream = torch.cuda.current_stream()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def batch(n, fn_name, steps=25):
+        torch.cuda.synchronize()
+        e0.record(stream)
+        for i in range(steps):
+            getattr(calls[n][i % kv_sets], fn_name)()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps * 1e3   # us per call
+
+    t_settle = time.perf_counter()
+    while (time.perf_counter() - t_settle) * 1e3 < args.settle_ms:
+        for n in names:
+            batch(n, "run", 8)
+    rounds = max(1, args.steps // 25)
+    whole, stage1 = {n: [] for n in names}, {n: [] for n in names}
+    for _ in range(rounds):
+        for n in names:
+            whole[n].append(batch(n, "run"))
+        for n in names:
+            stage1[n].append(batch(n, "run_stage1"))
+    med = lambda v: sorted(v)[len(v) // 2]
+    nbytes = algorithmic_bytes(cfg, x["kv_seq_len"].cpu(), mask_arg)
+    rows = {}
+    for n in names:
+        pl = calls[n][0].plan
+        rows[n] = {"us_per_call": round(med(whole[n]), 2), "stage1_us": round(med(stage1[n]), 2), "gbs": round(nbytes / med(whole[n]) / 1e3, 1),
+                   "plan": f"{pl.num_splits} x {pl.chunk_for(int(x['kv_seq_len'].max()))}", "rows_per_wg": pl.rows_per_wg, "mfma_loop": pl.mfma_loop}
+    print(json.dumps({"compare": {"workload": cfg.name, "batches_of_25_per_kernel": rounds, "kernels": rows}}))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -258,6 +312,10 @@ def main():
         kp[perm], vp[perm] = pool(kc), pool(vc)
         return kp, vp, perm.view(bsz, per_seq).to(torch.int32)
 
+    kernel_ids = {"auto": -1, "mfma": _lib.KERNEL_MFMA, "mfma_wide": _lib.KERNEL_MFMA_WIDE, "mfma_split_keys": _lib.KERNEL_MFMA_SPLIT_KEYS,
+                  "shuffle": _lib.KERNEL_SHUFFLE}
+    if args.compare:
+        return compare_kernels(args, cfg, x, mask_arg, [k.strip() for k in args.compare.split(",")], kernel_ids)
     calls = []
     for i, (kc, vc) in enumerate(zip(x["k_caches"], x["v_caches"])):
         tables = None
@@ -268,7 +326,7 @@ def main():
                 x["k_cache_paged"], x["v_cache_paged"], x["tables"] = kc, vc, tables
         calls.append(prepare(x["q"], kc, vc, x["current_k"], x["current_v"], mask_arg, x["kv_seq_len"], cfg.block_size,
                              None, None, None, None, x["sm_scale"], cfg.kv_group_num, _force_splits=args.splits,
-                             _force_kernel={"auto": -1, "mfma": _lib.KERNEL_MFMA, "mfma_wide": _lib.KERNEL_MFMA_WIDE, "mfma_split_keys": _lib.KERNEL_MFMA_SPLIT_KEYS, "shuffle": _lib.KERNEL_SHUFFLE}[args.kernel],
+                             _force_kernel=kernel_ids[args.kernel],
                              block_tables=tables))
     if args.paged:   # the contiguous copies are no longer needed, except set 0 for the self-check
         x["k_caches"], x["v_caches"] = x["k_caches"][:1], x["v_caches"][:1]
