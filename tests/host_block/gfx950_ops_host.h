@@ -46,17 +46,21 @@ inline WaveExchange& my_exchange() { return exchange()[threadIdx.x / 64]; }
 // Address of LDS byte `addr`, bounds-checked for an access of `bytes` bytes against what the launch asked for.
 // A direct global->LDS load of this lane that has not landed yet (late-landing mode).
 struct LoadInFlight {
-  const char* src;
+  const char* src;        // null: a load into registers (load_b128_device), its 16 bytes in `data`
   uint32_t lds_addr;
+  unsigned char data[16] = {};
 };
 inline bool& loads_land_late() { static bool late = std::getenv("FTA_HOST_LOADS_LAND_LATE") != nullptr; return late; }   // also host_block_loads_land_late()
 inline std::deque<LoadInFlight>& loads_in_flight() { static thread_local std::deque<LoadInFlight> q; return q; }
 inline char* lds_at(uint32_t addr, uint32_t bytes);
 // Lands the oldest loads of this lane until at most `allowed` are in flight (the counter retires in issue order).
+// Loads into registers that a wait has landed and no settle() has handed to its register yet, oldest first.
+inline std::deque<LoadInFlight>& landed_register_loads() { static thread_local std::deque<LoadInFlight> q; return q; }
 inline void land_all_but(size_t allowed) {
   std::deque<LoadInFlight>& q = loads_in_flight();
   while (q.size() > allowed) {
-    std::memcpy(lds_at(q.front().lds_addr, 16), q.front().src, 16);
+    if (q.front().src) std::memcpy(lds_at(q.front().lds_addr, 16), q.front().src, 16);
+    else landed_register_loads().push_back(q.front());
     q.pop_front();
   }
 }
@@ -68,6 +72,10 @@ inline std::deque<LdsReadInFlight>& lds_reads_in_flight() { static thread_local 
 inline void no_load_may_outlive_its_thread() {
   if (!loads_in_flight().empty()) {
     std::fprintf(stderr, "a thread left the kernel with %zu global->LDS loads in flight\n", loads_in_flight().size());
+    std::abort();
+  }
+  if (!landed_register_loads().empty()) {
+    std::fprintf(stderr, "a thread left the kernel with %zu loaded registers that no settle() took\n", landed_register_loads().size());
     std::abort();
   }
   if (!lds_reads_in_flight().empty()) {
@@ -201,7 +209,18 @@ template <int N> inline void wait_lgkm(u32x2& a, u32x2& b) {
   lds_reads::land_into(a);
   lds_reads::land_into(b);
 }
-inline void settle(f32x4&) {}
+// load_b128_device is a load the compiler does not see: the register holds nothing until a vmcnt wait has
+// landed the load (modelled in both load modes; with global->LDS loads that land when issued the count only
+// holds for vmcnt(0), the one wait the kernel uses for these), and settle() is where the kernel takes the value.
+inline void settle(f32x4& a) {
+  std::deque<host_block::LoadInFlight>& q = host_block::landed_register_loads();
+  if (q.empty()) {
+    std::fprintf(stderr, "settle() of a register whose load no vmcnt wait has landed\n");
+    std::abort();
+  }
+  std::memcpy(&a, q.front().data, 16);
+  q.pop_front();
+}
 
 template <int OFF>
 inline u32x4 lds_read_b128(uint32_t addr) {
@@ -227,8 +246,11 @@ inline u32x2 lds_read_tr16_b64(uint32_t addr) {
 
 inline void store_b128_device(void* ptr, f32x4 v) { std::memcpy(ptr, &v, 16); }
 inline f32x4 load_b128_device(const void* ptr) {
+  host_block::LoadInFlight load{nullptr, 0};
+  std::memcpy(load.data, ptr, 16);
+  host_block::loads_in_flight().push_back(load);
   f32x4 v;
-  std::memcpy(&v, ptr, 16);
+  std::memset(&v, 0xFF, 16);
   return v;
 }
 inline void scalar_load_one(const int32_t* p0, int& a0) { a0 = *p0; }
