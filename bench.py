@@ -267,6 +267,9 @@ def main():
     if args.gpus != 1:
         print("bench.py measures one GPU only: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
+    if args.steps < 1 or args.warmup < 0:
+        print("bench.py: --steps must be at least 1 and --warmup not negative", file=sys.stderr)
+        sys.exit(2)
     import torch
     from flash_tree_attn_amd import _lib, prepare
     from flash_tree_attn_amd.synthetic import CONFIGS, algorithmic_bytes, flops, make_inputs
@@ -362,14 +365,18 @@ def main():
         torch.cuda.synchronize()
     for i in range(args.warmup):
         calls[i % kv_sets].run()
-    # the timed region: exactly --steps calls, event-timed in batches of 25 (the last may be shorter). The headline is
-    # the median batch, so that one disturbed batch (a clock dip, another tenant of the host) does not move it; the
-    # mean over all steps is reported beside it.
-    sizes = [25] * (args.steps // 25) + ([args.steps % 25] if args.steps % 25 else [])
+    # the timed region: exactly --steps calls, event-timed in batches (25 calls each from 50 steps on, 5 each from 10
+    # on, one batch below that; the last batch takes what is left). With three batches or more the headline is the
+    # median batch, so that one disturbed batch (a clock dip, another tenant of the host) does not move it; with
+    # fewer it is the mean over all calls, and the line says which. The mean is reported beside it either way.
+    per_batch = 25 if args.steps >= 50 else 5 if args.steps >= 10 else args.steps
+    sizes = [per_batch] * (args.steps // per_batch) + ([args.steps % per_batch] if args.steps % per_batch else [])
     batch_ms = [timed("run", n) for n in sizes]
     ms_mean = sum(b * n for b, n in zip(batch_ms, sizes)) / args.steps
+    full = sorted(b for b, n in zip(batch_ms, sizes) if n == per_batch)   # a short last batch takes no part in the median
+    use_median = len(full) >= 3
+    ms = full[len(full) // 2] if use_median else ms_mean
     batch_sorted = sorted(batch_ms)
-    ms = batch_sorted[len(batch_sorted) // 2]
     single_launch = bool(plan.single_launch)   # the merge runs inside the stage-1 kernel
     ms_two = timed("run_two_launches", args.steps) if single_launch else ms
     ms_stage1_alone = timed("run_stage1", args.steps)
@@ -383,9 +390,11 @@ def main():
         "metric": "tree-attn us/call + achieved HBM GB/s (% peak), 8B GQA q_len=64 @8K ctx",
         "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "settle_ms": args.settle_ms, "ms_per_step": ms, "us_per_call": ms * 1e3,
-        "ms_per_step_is": "median of the event-timed batches of the --steps calls", "ms_per_step_mean": ms_mean,
-        "us_per_call_batches": {"median": round(ms * 1e3, 2), "min": round(batch_sorted[0] * 1e3, 2),
-                                "max": round(batch_sorted[-1] * 1e3, 2), "batches": len(sizes), "calls_per_batch": 25},
+        "ms_per_step_is": ("median of the event-timed batches of the --steps calls" if use_median else
+                           "mean over the --steps calls (fewer than three full batches: no median taken)"), "ms_per_step_mean": ms_mean,
+        "us_per_call_batches": {"median": round(full[len(full) // 2] * 1e3, 2) if use_median else None, "min": round(batch_sorted[0] * 1e3, 2),
+                                "max": round(batch_sorted[-1] * 1e3, 2), "batches": len(sizes), "calls_per_batch": per_batch,
+                                "calls_in_last_batch": sizes[-1]},
         "pct_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}[cfg.dtype],

@@ -139,11 +139,28 @@ __device__ __forceinline__ int block_max(int mine) {
   return __builtin_amdgcn_readfirstlane(m);
 }
 
+// Batches of up to 64 sequences: lane i of every wave takes sequence i's clamped length (0 beyond the
+// batch) and the wave finds the longest by itself, so that no wave waits for another.
+constexpr int kMaxWaveBatch = 64;
+__device__ __forceinline__ int wave_longest(const KernelParams& p, int* mine) {
+  const int lane = threadIdx.x & 63;
+  const int len = lane < p.bsz ? clamped_len(p, lane) : 0;
+  int m = len;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) m = max(m, __shfl_xor(m, o, 64));
+  *mine = len;
+  return __builtin_amdgcn_readfirstlane(m);
+}
+
 // Keys per split of this launch, from the lengths of the whole batch; every thread of the
 // block must call it, once per kernel. Every workgroup of stage 1 and of stage 2 computes
 // the same value from the same lengths, so no workgroup has to tell another.
 __device__ __forceinline__ int batch_chunk(const KernelParams& p) {
   if (p.bsz == 1) return chunk_for(p, clamped_len(p, 0));
+  if (p.bsz <= kMaxWaveBatch) {
+    int mine;
+    return chunk_for(p, wave_longest(p, &mine));
+  }
   int m = 0;
   for (int i = threadIdx.x; i < p.bsz; i += blockDim.x) m = max(m, clamped_len(p, i));
   return chunk_for(p, block_max(m));
@@ -156,10 +173,12 @@ __device__ __forceinline__ int batch_chunk(const KernelParams& p) {
 // first every full chunk (all equal work; sequence-major), then the last chunk of every
 // sequence (partial chunk + tree block) in descending size; what remains of the grid has
 // nothing to do. No host look at the lengths and no atomics: every workgroup recomputes
-// the order from the bsz lengths in LDS (and gets its sequence's clamped length and the
-// launch's chunk length back with it). Batches of one sequence or beyond
-// kMaxOrderedBatch keep the identity order. Returns false if the item is empty. Must be
-// called by all threads of the block.
+// the order from the bsz lengths (and gets its sequence's clamped length and the
+// launch's chunk length back with it). Batches of up to 64 sequences are resolved by every
+// wave on its own, in one pass over the lengths held one per lane, without LDS or barriers,
+// and in closed form when all sequences are equally long; larger ones up to kMaxOrderedBatch
+// go through LDS; batches of one sequence or beyond kMaxOrderedBatch keep the identity
+// order. Returns false if the item is empty. Must be called by all threads of the block.
 constexpr int kMaxOrderedBatch = 256;
 __device__ __forceinline__ bool item_by_order(const KernelParams& p, int k, int* batch, int* split, int* len, int* chunk_out) {
   if (p.bsz == 1 || p.bsz > kMaxOrderedBatch) {
@@ -168,6 +187,46 @@ __device__ __forceinline__ bool item_by_order(const KernelParams& p, int k, int*
     *batch = k / p.num_splits;
     *split = k % p.num_splits;
     *len = clamped_len(p, *batch);
+    return true;
+  }
+  if (p.bsz <= kMaxWaveBatch) {
+    const int lane = threadIdx.x & 63;
+    int my_len;
+    const int chunk = chunk_for(p, wave_longest(p, &my_len));
+    *chunk_out = chunk;
+    const bool in_batch = lane < p.bsz;
+    const int my_n = splits_for(my_len, chunk, p.num_splits);
+    const int my_full = in_batch ? my_n - 1 : 0;          // chunks of this sequence that are full
+    const int my_tail = my_len - (my_n - 1) * chunk;      // keys of its last chunk
+    const int len0 = __builtin_amdgcn_readlane(my_len, 0);
+    if (__builtin_amdgcn_ballot_w64(in_batch && my_len != len0) == 0) {
+      // equally long sequences: bsz * full chunks sequence-major, then the last chunks in batch order
+      const int full = __builtin_amdgcn_readlane(my_full, 0);
+      const int total = p.bsz * full;
+      *len = len0;
+      if (k < total) {
+        *batch = k / full;
+        *split = k % full;
+        return true;
+      }
+      *batch = k - total;
+      *split = full;
+      return k - total < p.bsz;
+    }
+    int before = 0, total = 0, rank = 0;
+    for (int j = 0; j < p.bsz; ++j) {
+      const int f = __builtin_amdgcn_readlane(my_full, j), t = __builtin_amdgcn_readlane(my_tail, j);
+      total += f;
+      before += j < lane ? f : 0;
+      rank += (t > my_tail) || (t == my_tail && j < lane);
+    }
+    const bool full = k >= before && k < before + my_full;
+    const uint64_t owner = __builtin_amdgcn_ballot_w64(in_batch && (full || k - total == rank));
+    if (owner == 0) return false;
+    const int src = __builtin_ctzll(owner);
+    *batch = src;
+    *split = __builtin_amdgcn_readlane(full ? k - before : my_n - 1, src);
+    *len = __builtin_amdgcn_readlane(my_len, src);
     return true;
   }
   __shared__ int s_nsp[kMaxOrderedBatch];

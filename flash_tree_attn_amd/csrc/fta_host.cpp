@@ -21,6 +21,7 @@ const EnvKnobs& env_knobs() {
     if (const char* e = std::getenv("FTA_TREE_TILE_WEIGHT")) k.tree_tile_weight = std::max(0, std::atoi(e));
     if (const char* e = std::getenv("FTA_WIDE_LOOP")) k.wide_loop = e[0] == '1';
     if (const char* e = std::getenv("FTA_SPLIT_KEYS")) k.split_keys = e[0] == '1';
+    if (const char* e = std::getenv("FTA_STAGE2_SHARED_WALK")) k.stage2_shared_walk = e[0] == '1';
     return k;
   }();
   return knobs;

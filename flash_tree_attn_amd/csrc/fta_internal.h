@@ -72,13 +72,15 @@ int launch_stage2_merge(const KernelParams& p, int dtype, int head_dim, void* st
 int mfma_rows_per_wg(int rows, int head_dim);
 
 // Tuning knobs from the environment, read once per process (comparison runs and tests only):
-// FTA_ROWS_PER_WG=128, FTA_FORCE_SPLITS=n, FTA_TREE_TILE_WEIGHT=n, FTA_WIDE_LOOP=1, FTA_SPLIT_KEYS=1.
+// FTA_ROWS_PER_WG=128, FTA_FORCE_SPLITS=n, FTA_TREE_TILE_WEIGHT=n, FTA_WIDE_LOOP=1, FTA_SPLIT_KEYS=1,
+// FTA_STAGE2_SHARED_WALK=1.
 struct EnvKnobs {
   bool rows_128;
   int force_splits;      // 0 = none
   int tree_tile_weight;  // < 0 = default
   bool wide_loop;
   bool split_keys;
+  bool stage2_shared_walk;   // stage 2: four threads share a row's walk over many splits (not yet timed against the plain walk)
 };
 const EnvKnobs& env_knobs();
 

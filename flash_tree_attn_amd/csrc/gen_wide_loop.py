@@ -534,15 +534,24 @@ def operands(D: int) -> str:
             f'"{{s{S_KTILE}}}"(w_ktile_lo)', f'"{{s{S_KTILE + 1}}}"(w_ktile_hi)', f'"{{s{S_VTILE}}}"(w_vtile_lo)', f'"{{s{S_VTILE + 1}}}"(w_vtile_hi)',
             f'"{{s{S_KDST}}}"(w_kdst)', f'"{{s{S_VDST}}}"(w_vdst)', f'"{{s{S_C}}}"(w_c)']
     clob = [f'"v{r}"' for r in list(range(V_S, V_VF + 4 * PF)) + list(range(V_PS, V_T + 6))]
-    clob += [f'"s{r}"' for r in range(S_TMP, S_TMP + 8)] + ['"vcc"', '"scc"', '"memory"']
+    # m0: the tile requests set it (the LDS destination of global_load_lds); the compiler's own requests around the
+    # statement use it too and must not assume a value across it
+    clob += [f'"s{r}"' for r in range(S_TMP, S_TMP + 8)] + ['"m0"', '"vcc"', '"scc"', '"memory"']
     return "      : " + ", ".join(outs) + "\n      : " + ", ".join(ins) + "\n      : " + ", ".join(clob)
+
+
+# scalar instructions that leave a result in SCC
+_SCC_WRITERS = ("s_add", "s_sub", "s_and_b", "s_or_b", "s_xor", "s_nand", "s_nor", "s_xnor", "s_lshl", "s_lshr", "s_ashr", "s_andn2", "s_orn2",
+                "s_min", "s_max", "s_abs", "s_bfe", "s_not", "s_bcnt")
 
 
 def verify(body: list[str], ops: str, name: str) -> None:
     """Raises if the assembly text touches a register the operand lists do not name. The compiler
     keeps its own values (addresses among them) in every register the statement does not
     declare, so an undeclared write is a wild pointer waiting to happen; an undeclared read is a
-    value nobody set. Also checks that register tuples start on an even register."""
+    value nobody set. The named registers (m0, vcc, scc, exec) are held to the same rule as the numbered ones: an
+    instruction that writes one, openly or by its definition (compares, scalar arithmetic), needs it among the
+    clobbers. Also checks that register tuples start on an even register."""
     import re
     decl = {"v": set(), "s": set(), "a": set()}
     inputs = {"v": set(), "s": set(), "a": set()}
@@ -550,6 +559,23 @@ def verify(body: list[str], ops: str, name: str) -> None:
         (decl if m.group(1) else inputs)[m.group(2)].add(int(m.group(3)))
     for m in re.finditer(r'"([vs])(\d+)"', ops.split("\n")[-1]):
         decl[m.group(1)].add(int(m.group(2)))
+    named_decl = set(re.findall(r'"(m0|vcc|scc|exec)"', ops.split("\n")[-1]))
+
+    def named_writes(op, arglist):
+        out = set()
+        if not op.startswith(("s_cbranch", "s_branch", "s_waitcnt", "s_nop", "s_barrier", "global_load_lds", "s_cmp")) and arglist:
+            head = arglist[0].split("_")[0]          # vcc_lo / exec_hi name a half of the pair
+            if head in ("m0", "vcc", "exec"):
+                out.add(head)
+        if op.startswith("v_cmp") and op.endswith("_e32"):
+            out.add("vcc")                           # the e32 form has no other destination
+        if op.startswith("v_cmpx"):
+            out.add("exec")
+        if op.startswith(("s_cmp", "s_bitcmp")) or op.startswith(_SCC_WRITERS):
+            out.add("scc")
+        if "saveexec" in op or op.startswith("s_wrexec"):
+            out.add("exec")
+        return out
 
     def regs(tok):
         for m in re.finditer(r"\b([vas])\[(\d+):(\d+)\]|\b([vas])(\d+)\b", tok):
@@ -583,6 +609,9 @@ def verify(body: list[str], ops: str, name: str) -> None:
                 bad = set(r) - decl[k]
                 if bad:
                     raise AssertionError(f"{name}: `{line}` writes undeclared {k}{sorted(bad)}")
+        bad_named = named_writes(op, arglist) - named_decl
+        if bad_named:
+            raise AssertionError(f"{name}: `{line}` writes undeclared {sorted(bad_named)}")
         for t in src:
             for k, r in regs(t):
                 bad = set(r) - decl[k] - inputs[k]
@@ -649,7 +678,7 @@ def hazards(body: list[str], name: str) -> None:
             if dist >= need:
                 return
 
-    scc_writers = ("s_add", "s_sub", "s_and_b", "s_or_b", "s_xor", "s_lshl", "s_lshr", "s_ashr", "s_andn2", "s_orn2", "s_min", "s_max", "s_abs", "s_bfe")
+    scc_writers = _SCC_WRITERS
     for i, (op, args, text) in enumerate(ins):
         d, _ = dst_src(op, args)
         if op.startswith("v_dot2c"):

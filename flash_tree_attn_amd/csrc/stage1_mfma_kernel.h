@@ -111,7 +111,11 @@ stage1_mfma_kernel(const KernelParams p) {
   constexpr int kLoadsPerTile = 2 * kLoadsPerTensor;
   constexpr int kRowsPerWave = 32 * QB;
   constexpr int kRowsPerWg = (KSPLIT ? NW / 2 : NW) * kRowsPerWave;
-  constexpr int kVRing = NSK * TL::kTileBytes;       // byte offset of the V ring
+  // K stages of the ring. Tiles are requested NSK ahead in every loop; the pipelined loop keeps one
+  // stage more, so that K of tile t is still in place behind iteration t, which may want its scores
+  // again (kHeavyShare), instead of being overwritten by the tile requested during that iteration.
+  constexpr int kKSlots = PIPE ? NSK + 1 : NSK;
+  constexpr int kVRing = kKSlots * TL::kTileBytes;   // byte offset of the V ring
 
   FTA_DYNAMIC_LDS(smem);
 
@@ -210,7 +214,7 @@ stage1_mfma_kernel(const KernelParams p) {
   // Ring slots of the next tile to go out (tiles go out in order, so the slots just count up and wrap).
   int k_slot = 0, v_slot = 0;
   auto advance_slots = [&]() __attribute__((always_inline)) {
-    k_slot = k_slot + 1 == NSK ? 0 : k_slot + 1;
+    k_slot = k_slot + 1 == kKSlots ? 0 : k_slot + 1;
     v_slot = v_slot + 1 == NSV ? 0 : v_slot + 1;
   };
   const int64_t k_wave_off = static_cast<int64_t>(wave * RPB) * k_row_bytes, v_wave_off = static_cast<int64_t>(wave * RPB) * v_row_bytes;
@@ -276,7 +280,8 @@ stage1_mfma_kernel(const KernelParams p) {
     }
   };
   // Tiles are requested in order. A tile may go out once the stage it lands in is free:
-  // tile j reuses the K stage of tile j-NSK and the V stage of tile j-NSV. `k_done` /
+  // tile j reuses the K stage of tile j-kKSlots and the V stage of tile j-NSV and goes out when
+  // tile j-NSK is done with (for the pipelined loop a stage later than it would have to). `k_done` /
   // `v_done` count the tiles whose K / V every wave has finished reading (as of the last
   // barrier).
   // `cap` bounds the tiles that may go out: ntiles normally; kPadRing lets the ring run
@@ -350,6 +355,14 @@ stage1_mfma_kernel(const KernelParams p) {
   f32x16 o[DB][QB];
   float m_run[QB], l_run[QB], alpha_pending[QB];
   bool rescale_pending = false;
+  // P goes into the second product rounded to T (flash_tree_attn.py:117). Where a single key carries a
+  // large share of a row's weight, that rounding (2^-9 relative for bf16) shows in the output, so a full
+  // tile whose largest probability exceeds kHeavyShare of the row's running sum takes the compensating
+  // product with the rounding residue as well, like every masked tile. The running sum only grows in
+  // units of the final maximum, so no key that ends up with that share of the row escapes. Each lane holds
+  // the sum of its part of the keys (half of them, a quarter with key halves); comparing against twice that
+  // errs on the side of compensating. The decision is one per wave and tile.
+  constexpr float kHeavyShare = 0.25f;
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
     m_run[qb] = neg_inf();
@@ -377,7 +390,7 @@ stage1_mfma_kernel(const KernelParams p) {
   // ---- building blocks -------------------------------------------------------------
   // S^T = K Q^T of tile t (fragment queue: kPF reads ahead of the consuming MFMA).
   auto qk_tile = [&](int t, f32x16 (&s)[2][QB]) __attribute__((always_inline)) {
-    const uint32_t ka = k_rd + (t % NSK) * TL::kTileBytes;
+    const uint32_t ka = k_rd + (t % kKSlots) * TL::kTileBytes;
     u32x4 kf[kKFrags];
     static_for<0, kPF>([&](auto f) { kf[f] = lds_read_b128<(f % 2) * kKbOff + (f / 2) * kKsOff>(ka); });
     static_for<0, kKFrags>([&](auto f) {
@@ -423,7 +436,7 @@ stage1_mfma_kernel(const KernelParams p) {
     constexpr int NV = HAS_PV ? kVFrags : 0;
     constexpr int NSTEP = NV + kKFrags;
     const uint32_t va = v_rd + ((t + NSV - 1) % NSV) * TL::kTileBytes;   // tile t-1
-    const uint32_t ka = k_rd + ((t + 1) % NSK) * TL::kTileBytes;         // tile t+1
+    const uint32_t ka = k_rd + ((t + 1) % kKSlots) * TL::kTileBytes;     // tile t+1
     u32x2 vlo[kVFrags], vhi[kVFrags];
     u32x4 kf[kKFrags];
     auto issue = [&](auto i) __attribute__((always_inline)) {
@@ -575,6 +588,42 @@ stage1_mfma_kernel(const KernelParams p) {
     }
     rescale_pending = wave_any(any_rescale);
   };
+  // Whether a full tile with the raw scores `s` holds a heavy key, decided ahead of its softmax (the
+  // unfused loops then send it through the masked softmax, which keeps the residue): the row's largest
+  // probability against what the lane will at least have summed, its running sum in the new units plus
+  // its own largest probability of the tile.
+  auto full_tile_is_heavy = [&](const f32x16 (&s)[2][QB]) __attribute__((always_inline)) {
+    bool any_heavy = false;
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+      float mx0 = fmaxf(s[0][qb][0], s[1][qb][0]), mx1 = fmaxf(s[0][qb][1], s[1][qb][1]);
+#pragma unroll
+      for (int r = 2; r < 16; r += 2) {
+        mx0 = fmaxf(mx0, fmaxf(s[0][qb][r], s[1][qb][r]));
+        mx1 = fmaxf(mx1, fmaxf(s[0][qb][r + 1], s[1][qb][r + 1]));
+      }
+      const float mx_lane = fmaxf(mx0, mx1), mx = half_swap_max(mx_lane, lh);
+      const float m_new = fmaxf(m_run[qb], mx * c);
+      const float p_top = fast_exp2(__builtin_fmaf(mx, c, -m_new)), p_lane = fast_exp2(__builtin_fmaf(mx_lane, c, -m_new));
+      any_heavy |= p_top > 2.f * kHeavyShare * __builtin_fmaf(l_run[qb], fast_exp2(m_run[qb] - m_new), p_lane);
+    }
+    return wave_any(any_heavy);
+  };
+  // The rounding residue of a full tile's probabilities `pf`, as a masked tile leaves it in `s`: the
+  // scores are computed again (K of the tile is still in its stage) and exponentiated against the
+  // running maximum, which is the one `pf` was made with.
+  auto residue_of_full_tile = [&](int t, f32x16 (&s)[2][QB], const Vec8 (&pf)[QB][4]) __attribute__((always_inline)) {
+    qk_tile(t, s);
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int kb = kk >> 1, r = (kk & 1) * 8 + e;
+          s[kb][qb][r] = fast_exp2(__builtin_fmaf(s[kb][qb][r], c, -m_run[qb])) - static_cast<float>(pf[qb][kk][e]);
+        }
+  };
   auto apply_rescale = [&]() __attribute__((always_inline)) {
     if (rescale_pending) {
 #pragma unroll
@@ -599,12 +648,18 @@ stage1_mfma_kernel(const KernelParams p) {
 
   // One fused iteration for full tile t: softmax(s_in) -> p_out on the vector ALU while
   // the matrix pipeline does P.V of tile t-1 (p_in, when HAS_PV) and K.Q of tile t+1 -> s_out.
-  auto fused = [&](auto has_pv_c, int t, f32x16 (&s_in)[2][QB], f32x16 (&s_out)[2][QB], const Vec8 (&p_in)[QB][4], Vec8 (&p_out)[QB][4]) __attribute__((always_inline)) {
+  auto fused = [&](auto has_pv_c, int t, f32x16 (&s_in)[2][QB], f32x16 (&s_out)[2][QB], Vec8 (&p_in)[QB][4], Vec8 (&p_out)[QB][4]) __attribute__((always_inline)) {
     // The lean softmax (full tile: no mask, no key limit) cut into slices, one per MFMA
     // step: steps [0, NA) take the row maximum, step NA exchanges it between the half
     // waves and fixes the new maximum, the following steps exponentiate and pack pairs
     // of values, the last step updates the running sum.
-    float mx0[QB], mx1[QB], m_new[QB], alpha[QB], ps0[QB], ps1[QB];
+    // The last slice also says whether the tile holds a heavy key (kHeavyShare): then the tile's
+    // scores are computed again (K of tile t stays in its stage for this, kKSlots), their rounding
+    // residue goes into the registers of the previous tile's probabilities, which the stream has
+    // consumed, and is multiplied with V of tile t, which landed with this iteration's
+    // synchronisation point. Nothing of this is live across the stream.
+    float mx0[QB], mx1[QB], m_new[QB], alpha[QB], ps0[QB], ps1[QB], p_top[QB];
+    bool heavy = false;
     auto slice = [&](auto i_c, auto nstep_c) __attribute__((always_inline)) {
       constexpr int I = decltype(i_c)::value, NSTEP = decltype(nstep_c)::value;
       constexpr int NA = NSTEP / 4, EPA = 32 / NA;
@@ -622,6 +677,7 @@ stage1_mfma_kernel(const KernelParams p) {
           const float mx = half_swap_max(fmaxf(mx0[qb], mx1[qb]), lh);
           m_new[qb] = fmaxf(m_run[qb], mx * c);
           alpha[qb] = fast_exp2(m_run[qb] - m_new[qb]);
+          p_top[qb] = fast_exp2(__builtin_fmaf(mx, c, -m_new[qb]));   // the row's largest probability of this tile
           ps0[qb] = 0.f;
           ps1[qb] = 0.f;
         } else {
@@ -640,25 +696,43 @@ stage1_mfma_kernel(const KernelParams p) {
         }
       }
       if constexpr (I == NSTEP - 1) {
-        bool any_rescale = false;
+        bool any_rescale = false, any_heavy = false;
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb) {
           l_run[qb] = l_run[qb] * alpha[qb] + (ps0[qb] + ps1[qb]);
           any_rescale |= m_new[qb] > m_run[qb];
+          any_heavy |= p_top[qb] > 2.f * kHeavyShare * l_run[qb];
           m_run[qb] = m_new[qb];
           alpha_pending[qb] = alpha[qb];
         }
         rescale_pending = wave_any(any_rescale);
+        heavy = wave_any(any_heavy);
       }
     };
     mma_stream(has_pv_c, t, p_in, s_out, slice);
+    if (heavy) {
+      apply_rescale();   // O in units of this tile's maximum before its residue is added
+      residue_of_full_tile(t, s_in, p_out);
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+          Vec8 pk;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) pk[e] = static_cast<T>(s_in[kk >> 1][qb][(kk & 1) * 8 + e]);
+          p_in[qb][kk] = pk;
+        }
+      pv_tile(t, p_in);
+    }
   };
 
-  // second, compensating P.V product of a masked tile: P's rounding residue is in `res`
-  auto pv_with_residue = [&](int tile, bool masked_tile, f32x16 (&res)[2][QB]) __attribute__((always_inline)) {
+  // P.V of a tile whose probabilities are in pA; a masked or heavy tile (`with_residue`) has left P's
+  // rounding residue in `res` and takes a second, compensating product with it. That one goes first:
+  // the 32 residue registers shrink to 16 before any product runs and are gone before the main one.
+  auto pv_with_residue = [&](int tile, bool with_residue, f32x16 (&res)[2][QB]) __attribute__((always_inline)) {
     apply_rescale();
     pv_tile(tile, pA);
-    if (masked_tile) {
+    if (with_residue) {
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
@@ -795,19 +869,32 @@ stage1_mfma_kernel(const KernelParams p) {
     }
     rescale_pending = wave_any(m_new > m_old);
   };
-  auto pv_half_with_residue = [&](int tile, bool masked_tile, const f32x16& res, Vec8 (&pf)[2]) __attribute__((always_inline)) {
+  auto half_tile_is_heavy = [&](const f32x16& s) __attribute__((always_inline)) {   // full_tile_is_heavy for one key block
+    float mx0 = s[0], mx1 = s[1];
+#pragma unroll
+    for (int r = 2; r < 16; r += 2) {
+      mx0 = fmaxf(mx0, s[r]);
+      mx1 = fmaxf(mx1, s[r + 1]);
+    }
+    const float mx_lane = fmaxf(mx0, mx1), mx = half_swap_max(mx_lane, lh);
+    const float m_new = fmaxf(m_run[0], mx * c);
+    const float p_top = fast_exp2(__builtin_fmaf(mx, c, -m_new)), p_lane = fast_exp2(__builtin_fmaf(mx_lane, c, -m_new));
+    return wave_any(p_top > 2.f * kHeavyShare * __builtin_fmaf(l_run[0], fast_exp2(m_run[0] - m_new), p_lane));
+  };
+  auto pv_half_with_residue = [&](int tile, bool with_residue, const f32x16& res, Vec8 (&pf)[2]) __attribute__((always_inline)) {
     apply_rescale();
-    pv_half(tile, pf);
-    if (masked_tile) {
+    if (with_residue) {   // the compensating product first, see pv_with_residue
+      Vec8 pr[2];
 #pragma unroll
       for (int kk = 0; kk < 2; ++kk) {
         Vec8 pk;
 #pragma unroll
         for (int e = 0; e < 8; ++e) pk[e] = static_cast<T>(res[kk * 8 + e]);
-        pf[kk] = pk;
+        pr[kk] = pk;
       }
-      pv_half(tile, pf);
+      pv_half(tile, pr);
     }
+    pv_half(tile, pf);
   };
 
 
@@ -916,9 +1003,10 @@ stage1_mfma_kernel(const KernelParams p) {
       const int key0 = tree ? t * kKeyTile : kv_start + (t - c0) * kKeyTile;
       if (tree) load_mask(key0, mask_vals);   // in flight while the scores are computed
       qk_tile(t, sB);
-      if (masked) softmax_tile(std::true_type{}, sB, pA, tree, key0, tree ? L : kv_end, mask_vals);
+      const bool with_residue = masked || full_tile_is_heavy(sB);   // (a full tile passes the key limit of the masked softmax whole)
+      if (with_residue) softmax_tile(std::true_type{}, sB, pA, tree, key0, tree ? L : kv_end, mask_vals);
       else softmax_tile(std::false_type{}, sB, pA, false, key0, kv_end, mask_vals);
-      pv_with_residue(t, masked, sB);
+      pv_with_residue(t, with_residue, sB);
     }
     if (!wave_active) return;
   } else if constexpr (KSPLIT) {
@@ -929,10 +1017,12 @@ stage1_mfma_kernel(const KernelParams p) {
       sync_point(t, t, t, ntiles);
       if (!wave_active) continue;
       const bool tree = t < tree_tiles;
-      const bool masked = tree || t - c0 >= full_tiles;
       const int key0 = (tree ? t * kKeyTile : kv_start + (t - c0) * kKeyTile) + 32 * kb_own;
       if (tree) load_mask_half(key0, mask_half);   // in flight while the scores are computed
       qk_half(t, s_half);
+      // tree and ragged tiles, and full tiles in which this wave's 32 keys hold a heavy one (against the
+      // wave's own running sum: its partner's keys only add to the row's), keep the residue
+      const bool masked = tree || t - c0 >= full_tiles || half_tile_is_heavy(s_half);
       if (masked) softmax_half(std::true_type{}, s_half, p_half, tree, key0, tree ? L : kv_end, mask_half);
       else softmax_half(std::false_type{}, s_half, p_half, false, key0, kv_end, mask_half);
       pv_half_with_residue(t, masked, s_half, p_half);
@@ -1029,10 +1119,16 @@ stage1_mfma_kernel(const KernelParams p) {
         const uint32_t w_vstep_lo = static_cast<uint32_t>(v_step), w_vstep_hi = static_cast<uint32_t>(static_cast<uint64_t>(v_step) >> 32);
         const uint32_t w_krd = k_rd, w_vrd = v_rd, w_koff = k_lane_off, w_voff = v_lane_off;
         const float w_c = c;
+        // The statement names M0 among its clobbers (its tile requests set it): the compiler never keeps a
+        // value of its own there, which is all its warning about reserved registers says, but it does merge
+        // and hoist the M0 writes of its own requests around the statement and must see this one.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
         if constexpr (D == 128 && std::is_same<T, __bf16>::value) FTA_WIDE_LOOP_128_BF16();
         else if constexpr (D == 128) FTA_WIDE_LOOP_128_F16();
         else if constexpr (std::is_same<T, __bf16>::value) FTA_WIDE_LOOP_64_BF16();
         else FTA_WIDE_LOOP_64_F16();
+#pragma clang diagnostic pop
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb) {
 #pragma unroll
@@ -1132,8 +1228,8 @@ stage1_mfma_kernel(const KernelParams p) {
     for (; t < ntiles; ++t) {
       sync_point(t + 1 < ntiles ? t + 1 : -1, t + 1, max(c0, t - 1), ntiles);
       if (!wave_active) continue;
-      const bool masked = t - c0 >= full_tiles;
       if (pv_pending) pv_with_residue(t - 1, prv_masked, sA);
+      const bool masked = t - c0 >= full_tiles || full_tile_is_heavy(sB);   // ragged, or a heavy key: the residue is kept
       if (masked) softmax_tile(std::true_type{}, sB, pA, false, kv_start + (t - c0) * kKeyTile, kv_end, mask_vals);
       else softmax_tile(std::false_type{}, sB, pA, false, kv_start + (t - c0) * kKeyTile, kv_end, mask_vals);
       // a masked tile leaves the rounding residue of P in sB: park it in sA, the scores of
@@ -1284,8 +1380,8 @@ stage1_mfma_kernel(const KernelParams p) {
 
 template <typename T, int D, int QB, int NW, int NS, int MODE, bool PAGED>
 int launch(const KernelParams& p, hipStream_t stream) {
-  // K ring of NS stages + V ring of NS (+ 2 pipelined, + 1 half-tile pipeline)
-  constexpr int kSmem = (MODE == kPipelined ? 2 * NS + 2 : MODE == kWide ? 2 * NS + 1 : 2 * NS) * TileLayout<D>::kTileBytes;   // kPlain, kSplitKeys: 2 * NS
+  // K ring of NS stages (+ 1 pipelined) + V ring of NS (+ 2 pipelined, + 1 half-tile pipeline)
+  constexpr int kSmem = (MODE == kPipelined ? 2 * NS + 3 : MODE == kWide ? 2 * NS + 1 : 2 * NS) * TileLayout<D>::kTileBytes;   // kPlain, kSplitKeys: 2 * NS
   static_assert(kSmem + 3 * 1024 <= 160 * 1024, "LDS budget (rings + the static arrays of item_by_order)");
   auto kern = stage1_mfma_kernel<T, D, QB, NW, NS, MODE, PAGED>;
   if (kSmem > 64 * 1024) {

@@ -4,8 +4,8 @@
 //
 // One thread owns four consecutive head_dim columns of one output row; the row's
 // split weights exp(lse_s - max) are recomputed per thread (the split count is
-// small by construction of the heuristic). With many splits and few rows four
-// threads share the walk over the splits (see the kernel).
+// small by construction of the heuristic). On request, with many splits and few rows,
+// four threads share the walk over the splits (see the kernel and launch()).
 #include "fta_device.h"
 
 namespace fta {
@@ -98,10 +98,11 @@ int launch_sg(const KernelParams& p, hipStream_t stream) {
 
 template <typename T, int D>
 int launch(const KernelParams& p, hipStream_t stream) {
-  // Waves the one-thread-per-column form would launch: below 16 per CU of a 256-CU part, with eight splits or
-  // more to walk, the walk is shared by four threads.
+  // The shared walk is for launches that would otherwise leave the machine few waves with long walks: fewer
+  // than 16 waves per CU of a 256-CU part in the one-thread-per-column form, eight splits or more. It has not
+  // been timed against the plain walk yet, so it only runs on request (FTA_STAGE2_SHARED_WALK=1).
   const int64_t waves = static_cast<int64_t>(p.bsz) * p.num_q_heads * p.q_len * (D / 4) / 64;
-  if (p.num_splits >= 8 && waves < 16 * kDefaultCUs) return launch_sg<T, D, 4>(p, stream);
+  if (env_knobs().stage2_shared_walk && p.num_splits >= 8 && waves < 16 * kDefaultCUs) return launch_sg<T, D, 4>(p, stream);
   return launch_sg<T, D, 1>(p, stream);
 }
 

@@ -1,6 +1,6 @@
 // Host stand-in for the HIP names that the simpler kernels of this library use, so that their source
 // runs on the CPU exactly as written: one host thread per GPU thread, std::barrier for __syncthreads,
-// an exchange array per wave for __shfl_xor, a plain buffer for the dynamic LDS, and hipLaunchKernel
+// an exchange array per wave for __shfl_xor / ballot / readlane, a plain buffer for the dynamic LDS, and hipLaunchKernel
 // = "run the grid, one workgroup after the other". TEST INFRASTRUCTURE ONLY: nothing under
 // flash_tree_attn_amd/ includes or loads this; it exists so that device code can be checked against the
 // oracle where no GPU is at hand (tests/test_dispatch_host.py, tests/test_host_block_kernels.py). Kernels
@@ -93,6 +93,25 @@ inline int host_readfirstlane(int v) {
   return first;
 }
 #define __builtin_amdgcn_readfirstlane(x) host_readfirstlane(x)
+// One bit per lane of the wave that holds `pred` (lanes the block does not have read as 0).
+inline uint64_t host_ballot(bool pred) {
+  host_block::Block& b = *host_block::current();
+  const unsigned t = threadIdx.x, w = t / 64;
+  b.slot[t] = pred ? 1u : 0u;
+  b.wave[w]->arrive_and_wait();
+  uint64_t bits = 0;
+  for (unsigned l = 0; l < 64 && 64 * w + l < b.threads; ++l) bits |= static_cast<uint64_t>(b.slot[64 * w + l]) << l;
+  b.wave[w]->arrive_and_wait();
+  return bits;
+}
+#define __builtin_amdgcn_ballot_w64(pred) host_ballot(pred)
+// Value of lane `sel` of the wave. The instruction takes the lane from a scalar register: the stand-in holds
+// the callers to a selector that is the same in every lane.
+inline int host_readlane(int v, int sel) {
+  if (host_readfirstlane(sel) != sel || sel < 0 || sel > 63) std::abort();
+  return __shfl_xor(v, static_cast<int>(threadIdx.x & 63) ^ sel, 64);   // lane ^ (lane ^ sel) = sel
+}
+#define __builtin_amdgcn_readlane(v, sel) host_readlane(v, sel)
 #define __builtin_amdgcn_exp2f(x) exp2f(x)
 #define __builtin_amdgcn_logf(x) log2f(x)
 #define __builtin_amdgcn_fence(order, scope) ((void)0)

@@ -51,6 +51,13 @@ def host_lib(tmp_path_factory):
     lib.fta_plan.argtypes = [C.POINTER(_lib.FtaArgs), C.c_int, C.POINTER(_lib.FtaPlanOut)]
     lib.fta_append_kv.argtypes = [C.POINTER(_lib.FtaAppendArgs), C.c_void_p]
     assert lib.fta_abi_version() == _lib.ABI_VERSION
+    # This copy of the library runs stage 2's shared walk where it applies (the product only does on request): the
+    # knobs are read once, by the first plan, so the request only has to stand until then.
+    os.environ["FTA_STAGE2_SHARED_WALK"] = "1"
+    try:
+        HostCall(lib, make(0, 1, 1, 1, 1, 32, 64, torch.float32, [64]))
+    finally:
+        del os.environ["FTA_STAGE2_SHARED_WALK"]
     return lib
 
 

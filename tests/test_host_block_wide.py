@@ -141,6 +141,25 @@ def test_64_row_wave_kernel_on_host_threads(host_lib, case):
         torch.testing.assert_close(out.float(), narrow.run().float(), **TOL[dtype])
 
 
+# Keys of more spread than N(0, 1): a few keys carry each row. The loop's lazy softmax exponentiates against a stale
+# reference, so every probability of a row, its largest included, is rounded to bf16 (2^-9 relative) where the other
+# loops hold the largest exactly at 1, and full tiles take no compensating product with the rounding residue (the
+# 8-wave, 4-wave and key-halves loops do: tests/test_host_block_mfma.py). At twice the spread the loop stays inside
+# the tolerance; at four times it does not (1.06 - 1.42 of atol 2e-3 / rtol 1e-2 here, 3 of 32768 values beyond it
+# on the GPU at 1024 keys). That is a known limit of this opt-in loop: the rows stay here, marked, until it is lifted.
+@pytest.mark.parametrize("scale_k,seed,keys", [
+    (2.0, 0, 512), (2.0, 3, 512), (2.0, 75, 1024),
+    pytest.param(4.0, 0, 512, marks=pytest.mark.xfail(strict=True, reason="known limit: bf16 probabilities of peaked rows, no residue product in the assembly loop")),
+    pytest.param(4.0, 3, 512, marks=pytest.mark.xfail(strict=True, reason="known limit: bf16 probabilities of peaked rows, no residue product in the assembly loop")),
+])
+def test_64_row_wave_kernel_on_peaked_rows(host_lib, scale_k, seed, keys):
+    x = make(seed, 1, 4, 1, 64, 128, keys, torch.bfloat16, [keys])
+    x["k_cache"] = (x["k_cache"].float() * scale_k).to(torch.bfloat16)
+    call = HostCall(host_lib, x, splits=1, kernel=WIDE)
+    assert call.plan.mfma_loop == 1
+    torch.testing.assert_close(call.run().float(), oracle(x), **TOL[torch.bfloat16])
+
+
 def test_64_row_wave_kernel_partials_and_merge_inside_the_launch(host_lib):
     lens, tmax, S = [330, 0], 2048, 3
     x = make(77, 2, 3, 1, 64, 128, tmax, torch.bfloat16, lens)

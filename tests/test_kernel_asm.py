@@ -213,6 +213,14 @@ def test_generator_rejects_undeclared_registers():
     # register tuples of vector registers start on an even register
     with pytest.raises(AssertionError, match="misaligned"):
         gen.verify(body + [f"v_mov_b64 v[{gen.V_T + 0 | 1}:{(gen.V_T + 0 | 1) + 1}], 0"], ops, "odd tuple")
+    # the named registers are held to the same rule: M0 (the LDS destination of the tile requests; the compiler's
+    # own requests around the statement use it as well), VCC (vector compares), SCC (scalar compares and arithmetic)
+    for named, what in (("m0", "s_mov_b32 m0"), ("vcc", "v_cmp"), ("scc", "s_")):
+        assert f'"{named}"' in ops and any(l.startswith(what) for l in body)
+        with pytest.raises(AssertionError, match=rf"writes undeclared \['{named}'\]"):
+            gen.verify(body, ops.replace(f'"{named}", ', ""), "named clobber dropped")
+    with pytest.raises(AssertionError, match=r"writes undeclared \['exec'\]"):
+        gen.verify(body + ["s_and_saveexec_b64 s[86:87], vcc"], ops, "exec written")
     # the masked-half statements go through the same check
     for H in (0, 1):
         gen.verify(gen.gen_masked(64, "f16", H), gen.operands_masked(64), "masked")

@@ -16,6 +16,11 @@ def test_more_than_one_gpu_is_refused_with_a_message():
     assert r.returncode != 0 and "one GPU" in r.stderr and r.stdout.strip() == ""
 
 
+def test_no_steps_is_refused_with_a_message():
+    r = subprocess.run([sys.executable, BENCH, "--steps", "0"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0 and "--steps" in r.stderr and r.stdout.strip() == ""
+
+
 def test_workloads_named_by_the_bench_exist():
     from flash_tree_attn_amd.synthetic import CONFIGS, algorithmic_bytes
     import torch
@@ -48,3 +53,7 @@ def test_json_line_of_a_short_run():
     cb = d["cpu_baseline"]
     assert cb["kind"] == "port" and cb["unit"] == "GB/s" and cb["cores"] >= 1 and cb["value"] > 0 and "sample" in cb
     assert abs(d["value"] - d["config"]["algorithmic_bytes"] / (d["ms_per_step"] * 1e-3) / 1e9) < 1.0
+    # 20 steps are four batches of five calls, and the line says so
+    bt = d["us_per_call_batches"]
+    assert bt["batches"] == 4 and bt["calls_per_batch"] == 5 and bt["calls_in_last_batch"] == 5 and "median" in d["ms_per_step_is"]
+    assert bt["min"] <= bt["median"] <= bt["max"]
