@@ -117,8 +117,8 @@ int plan(const fta_args& a, int num_cus, fta_plan_out* out) {
   const bool split_keys = split_ok && (a.force_kernel == FTA_KERNEL_MFMA_SPLIT_KEYS || (a.force_kernel < 0 && env_knobs().split_keys));
   const int rows_per_wg = kernel != FTA_KERNEL_MFMA ? 16 : split_keys ? 64 : mfma_rows_per_wg(rows, a.head_dim);
   // The 64-row-wave loop serves 256-row workgroups on contiguous caches, head_dim 64 / 128. It is
-  // opt-in (force_kernel or FTA_WIDE_LOOP=1): at the headline shape it measures level with the
-  // 8-wave loop, ahead of it on long chunks and behind it on short ones.
+  // opt-in (force_kernel or FTA_WIDE_LOOP=1): its one recorded timing at the headline shape is 5 % behind
+  // the 8-wave loop, and bf16 rows carried by a few keys exceed the tolerance in it.
   const bool wide_ok = kernel == FTA_KERNEL_MFMA && rows_per_wg == 256 && !a.block_table && a.head_dim <= 128;
   if (a.force_kernel == FTA_KERNEL_MFMA_WIDE && !wide_ok) return FTA_ERR_UNSUPPORTED;
   const bool wide = wide_ok && (a.force_kernel == FTA_KERNEL_MFMA_WIDE || (a.force_kernel < 0 && env_knobs().wide_loop));
@@ -194,9 +194,9 @@ int plan(const fta_args& a, int num_cus, fta_plan_out* out) {
     // latency-bound step worth about three cache tiles per tree tile): count it as extra
     // keys when cutting chunks, so that the last split of a full-length sequence gets a
     // correspondingly shorter cache range.
-    // The 64-row-wave loop runs its cache tiles faster (1.9-2.1 us against 2.36) and its tree tiles slower
-    // (unpipelined masked halves, 13-16 us per tree tile in the kernel's own clock reads): 7 tiles' worth.
-    const int64_t tree_weight = env_knobs().tree_tile_weight >= 0 ? env_knobs().tree_tile_weight : wide ? 7 : 3;
+    // (The 64-row-wave loop's unpipelined masked halves probably weigh more; until a timing says how much it is cut
+    // like the 8-wave loop. FTA_TREE_TILE_WEIGHT sets the weight for such a run.)
+    const int64_t tree_weight = env_knobs().tree_tile_weight >= 0 ? env_knobs().tree_tile_weight : 3;
     const int64_t tree_keys = splits > 1 ? tree_weight * kKeyTile * cdiv(a.q_len, kKeyTile) : 0;
     int64_t chunk = cdiv(cdiv(t_len + tree_keys, splits), gran) * gran;
     if ((splits - 1) * chunk >= t_len) chunk = cdiv(cdiv(t_len, splits), gran) * gran;

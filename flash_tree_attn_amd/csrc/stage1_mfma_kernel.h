@@ -34,10 +34,10 @@
 // a sequence last merges the partials itself (flash_tree_attn.py:339-365).
 //
 // Two loop variants: 8 waves / 256 rows with a software pipeline (softmax of tile t
-// sliced behind the MFMAs of P.V(t-1) and K.Q(t+1), K ring 3 / V ring 5, one workgroup
-// per CU), and 4 waves / 128 rows with a plain loop and rings of 2 so that two
-// workgroups share a CU (head_dim 256 only has this variant, alone on its CU: its tiles are
-// twice as large). Caches are contiguous per sequence or paged through a block
+// sliced behind the MFMAs of P.V(t-1) and K.Q(t+1), K requested 3 tiles ahead into a
+// ring of 4 stages / V ring 5, one workgroup per CU), and 4 waves / 128 rows with a plain
+// loop and rings of 2 so that two workgroups share a CU (head_dim 256 only has this
+// variant, alone on its CU: its tiles are twice as large). Caches are contiguous per sequence or paged through a block
 // table (a template parameter, so that the contiguous path carries no lookups).
 #pragma once
 #include <cstdlib>

@@ -44,8 +44,8 @@ struct Block {
   unsigned threads;
   std::barrier<> all;
   std::vector<std::unique_ptr<std::barrier<>>> wave;
-  std::vector<uint32_t> slot;
-  explicit Block(unsigned n) : threads(n), all(n), slot(n) {
+  std::vector<uint32_t> slot, slot2;
+  explicit Block(unsigned n) : threads(n), all(n), slot(n), slot2(n) {
     for (unsigned w = 0; w < (n + 63) / 64; ++w) wave.emplace_back(new std::barrier<>(std::min(64u, n - 64 * w)));
   }
 };
@@ -108,8 +108,19 @@ inline uint64_t host_ballot(bool pred) {
 // Value of lane `sel` of the wave. The instruction takes the lane from a scalar register: the stand-in holds
 // the callers to a selector that is the same in every lane.
 inline int host_readlane(int v, int sel) {
-  if (host_readfirstlane(sel) != sel || sel < 0 || sel > 63) std::abort();
-  return __shfl_xor(v, static_cast<int>(threadIdx.x & 63) ^ sel, 64);   // lane ^ (lane ^ sel) = sel
+  host_block::Block& b = *host_block::current();
+  const unsigned t = threadIdx.x, w = t / 64;
+  std::memcpy(&b.slot[t], &v, 4);
+  b.slot2[t] = static_cast<uint32_t>(sel);
+  b.wave[w]->arrive_and_wait();
+  if (sel < 0 || sel > 63 || b.slot2[64 * w] != static_cast<uint32_t>(sel)) {
+    std::fprintf(stderr, "readlane with a lane selector that differs between lanes\n");
+    std::abort();
+  }
+  int r;
+  std::memcpy(&r, &b.slot[64 * w + static_cast<unsigned>(sel)], 4);
+  b.wave[w]->arrive_and_wait();
+  return r;
 }
 #define __builtin_amdgcn_readlane(v, sel) host_readlane(v, sel)
 #define __builtin_amdgcn_exp2f(x) exp2f(x)

@@ -276,8 +276,8 @@ def test_plan_of_the_64_row_wave_loop(fta_lib):
     wide = dict(num_q_heads=32, num_kv_heads=8, cur_heads=8, q_len=64, force_kernel=_lib.KERNEL_MFMA_WIDE)
     st, pl = plan(fta_lib, base_args(**wide))
     assert st == 0 and pl.kernel == _lib.KERNEL_MFMA and pl.rows_per_wg == 256 and pl.mfma_loop == 1
-    # its tree tiles cost more and its cache tiles less than the 8-wave loop's: the split that owns the tree gets a shorter cache range
-    assert (pl.num_splits, pl.chunk) == (4, 2176)
+    # cut like the 8-wave loop until a timing of its tree phase says otherwise (FTA_TREE_TILE_WEIGHT sets the weight for such a run)
+    assert (pl.num_splits, pl.chunk) == (4, 2112)
     st, pl = plan(fta_lib, base_args(**{**wide, "force_kernel": _lib.KERNEL_MFMA}))
     assert st == 0 and pl.rows_per_wg == 256 and pl.mfma_loop == 0
     if not os.environ.get("FTA_WIDE_LOOP"):

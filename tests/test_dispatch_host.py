@@ -99,9 +99,9 @@ def test_dispatch_functions_as_compiled_cpp(fta_lib, runner):
     add([5000], 256, cache_len=65536, v_cache_len=65536)                               # one sequence: no ordering pass
     add([0], 512, cache_len=4096, v_cache_len=4096)
     add([4096, 9999, -5, 4095], 256, cache_len=4096, v_cache_len=4096, force_splits=3)  # clamped to the cache, negative = empty
-    add([rng.randrange(0, 3000) for _ in range(37)], 256, cache_len=4096, v_cache_len=4096, force_splits=3)
-    add([(37 * i) % 400 for i in range(300)], 256, cache_len=4096, v_cache_len=4096, force_splits=2)   # beyond the ordered limit
-    add([rng.randrange(0, 33000) for _ in range(64)], 64, cache_len=32768, v_cache_len=32768, force_splits=3)    # the largest batch a wave orders by itself
+    add([rng.randrange(0, 3000) for _ in range(19)], 64, cache_len=4096, v_cache_len=4096, force_splits=3)
+    add([(37 * i) % 400 for i in range(257)], 64, cache_len=4096, v_cache_len=4096, force_splits=2)   # beyond the ordered limit
+    add([rng.randrange(0, 33000) for _ in range(64)], 64, cache_len=32768, v_cache_len=32768, force_splits=2)    # the largest batch a wave orders by itself
     add([rng.randrange(0, 3000) for _ in range(65)], 128, cache_len=4096, v_cache_len=4096, force_splits=3)      # the smallest that goes through LDS
     add([100] * 6, 256, cache_len=4096, v_cache_len=4096, force_splits=4)                  # equally long, one live split each: the closed form without full chunks
     add([0] * 3, 512, cache_len=4096, v_cache_len=4096, force_splits=2)                    # nothing cached anywhere
