@@ -37,8 +37,9 @@
 // sliced behind the MFMAs of P.V(t-1) and K.Q(t+1), K requested 3 tiles ahead into a
 // ring of 4 stages / V ring 5, one workgroup per CU), and 4 waves / 128 rows with a plain
 // loop and rings of 2 so that two workgroups share a CU (head_dim 256 only has this
-// variant, alone on its CU: its tiles are twice as large). Caches are contiguous per sequence or paged through a block
-// table (a template parameter, so that the contiguous path carries no lookups).
+// variant, alone on its CU: its tiles are twice as large). Caches are contiguous per
+// sequence or paged through a block table (a template parameter, so that the contiguous
+// path carries no lookups).
 #pragma once
 #include <cstdlib>
 #include <type_traits>
@@ -727,8 +728,8 @@ stage1_mfma_kernel(const KernelParams p) {
   };
 
   // P.V of a tile whose probabilities are in pA; a masked or heavy tile (`with_residue`) has left P's
-  // rounding residue in `res` and takes a second, compensating product with it. That one goes first:
-  // the 32 residue registers shrink to 16 before any product runs and are gone before the main one.
+  // rounding residue in `res` and takes a second, compensating product with it (packed into pA once the
+  // main product has read it).
   auto pv_with_residue = [&](int tile, bool with_residue, f32x16 (&res)[2][QB]) __attribute__((always_inline)) {
     apply_rescale();
     pv_tile(tile, pA);
@@ -883,7 +884,7 @@ stage1_mfma_kernel(const KernelParams p) {
   };
   auto pv_half_with_residue = [&](int tile, bool with_residue, const f32x16& res, Vec8 (&pf)[2]) __attribute__((always_inline)) {
     apply_rescale();
-    if (with_residue) {   // the compensating product first, see pv_with_residue
+    if (with_residue) {   // the compensating product, first: the residue's 16 registers shrink to 4 before any product runs
       Vec8 pr[2];
 #pragma unroll
       for (int kk = 0; kk < 2; ++kk) {
