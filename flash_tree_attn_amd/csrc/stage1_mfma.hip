@@ -14,7 +14,7 @@ template <typename T, bool PAGED>
 int launch_t(const KernelParams& p, int head_dim, hipStream_t stream) {
   if (p.rows_per_wg == 256) {
     // 4 waves x 64 rows with the half-tile pipeline (stage1_mfma_wide.hip), or
-    // 8 waves x 32 rows, pipelined over whole tiles, K ring 3 / V ring 5; one workgroup per CU either way
+    // 8 waves x 32 rows, pipelined over whole tiles, K requested 3 tiles ahead into 4 stages / V ring 5; one workgroup per CU either way
     if (p.wide_loop && !PAGED) return launch_stage1_mfma_wide(p, dtype_of(T{}), head_dim, stream);
     if (head_dim == 128) return launch<T, 128, 1, 8, 3, kPipelined, PAGED>(p, stream);
     if (head_dim == 64) return launch<T, 64, 1, 8, 3, kPipelined, PAGED>(p, stream);

@@ -86,8 +86,9 @@ constexpr int kPipelined = 1;   // 8 waves x 32 rows, software pipeline over who
 constexpr int kWide = 2;        // 4 waves x 64 rows, software pipeline over half tiles, one wave per SIMD
 constexpr int kSplitKeys = 3;   // 4 waves, 64 rows: like kPlain, but two waves share a 32-row block, each taking 32 of a tile's 64 keys
 
-// NSK >= 2: K of tile t+1 is read during iteration t and must have been requested an
-// iteration earlier.
+// NSK: how many tiles ahead K is requested. NSK >= 2: K of tile t+1 is read during iteration t
+// and must have been requested an iteration earlier. (The K ring has NSK stages, one more in
+// the pipelined loop: kKSlots.)
 template <typename T, int D, int QB, int NW, int NSK, int MODE, bool PAGED>
 __global__ void __launch_bounds__(NW * 64)
 FTA_WAVES_PER_EU(((QB == 1 && D <= 128) ? 2 : 1))   // head_dim 256 and 64-row waves need the whole register file

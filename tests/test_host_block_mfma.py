@@ -301,7 +301,7 @@ def test_key_halves_are_refused_where_they_do_not_exist(host_lib):
 
 @pytest.mark.parametrize("shape", [
     # bsz hq hkv L  D    tmax dtype           lens         splits kernel      rows_per_wg
-    (1, 8, 1, 20, 128, 512, torch.float16, [470], 1, MFMA, 256),                 # the 8-wave pipeline: K ring 3, V ring 5, waits of 1 .. 4 tiles
+    (1, 8, 1, 20, 128, 512, torch.float16, [470], 1, MFMA, 256),                 # the 8-wave pipeline: K 3 tiles ahead in 4 stages, V ring 5, waits of 1 .. 4 tiles
     (1, 8, 1, 20, 128, 256, torch.bfloat16, [70], 1, MFMA, 256),                 # the same with fewer tiles than its rings hold
     (2, 4, 4, 26, 128, 320, torch.float16, [300, 64], 3, SPLIT_KEYS, 64),        # key halves
 ])

@@ -147,7 +147,7 @@ def test_the_whole_tile_pipelined_loop_has_no_spill_traffic(kernels):
     wait longer than intended (never shorter: the counter retires in order)."""
     checked = 0
     for name, (ins, _) in kernels.items():
-        if "Li1ELi8ELi3ELi1ELb" not in name:   # <.., 32-row waves, 8 waves, K ring 3, pipelined, ..>
+        if "Li1ELi8ELi3ELi1ELb" not in name:   # <.., 32-row waves, 8 waves, K requested 3 ahead, pipelined, ..>
             continue
         blocks, cur = [], []
         for l in ins:
