@@ -61,10 +61,11 @@ def host_lib(tmp_path_factory):
     return lib
 
 
-def make(seed, bsz, hq, hkv, L, D, tmax, dtype, lens):
+def make(seed, bsz, hq, hkv, L, D, tmax, dtype, lens, cur_heads=None):
     g = torch.Generator().manual_seed(seed)
     r = lambda *s: torch.randn(*s, generator=g).to(dtype)
-    x = dict(q=r(bsz, hq, L, D), k_cache=r(bsz, hkv, tmax, D), v_cache=r(bsz, hkv, tmax, D), current_k=r(bsz, hkv, L, D), current_v=r(bsz, hkv, L, D))
+    ch = hkv if cur_heads is None else cur_heads      # tree K/V per cache head (the default) or per query head
+    x = dict(q=r(bsz, hq, L, D), k_cache=r(bsz, hkv, tmax, D), v_cache=r(bsz, hkv, tmax, D), current_k=r(bsz, ch, L, D), current_v=r(bsz, ch, L, D))
     x["mask"] = additive_mask_from_parents(random_tree_parents(L, g), device="cpu")
     x["kv_seq_len"] = torch.as_tensor(lens, dtype=torch.int64)
     x["kv_group_num"] = hq // hkv
@@ -74,7 +75,7 @@ def make(seed, bsz, hq, hkv, L, D, tmax, dtype, lens):
 class HostCall:
     """fta_args over CPU tensors (what flash_decoding.prepare does for device tensors), planned, with scratch."""
 
-    def __init__(self, lib, x, splits=0, hint=0, mask=None, tables=None, pools=None, kernel=_lib.KERNEL_SHUFFLE, counters=False):
+    def __init__(self, lib, x, splits=0, hint=0, mask=None, tables=None, pools=None, kernel=_lib.KERNEL_SHUFFLE, counters=False, block_size=64, len32=False):
         self.lib, self.x = lib, x
         q = x["q"]
         bsz, hq, L, D = q.shape
@@ -82,9 +83,10 @@ class HostCall:
         mask = x["mask"] if mask is None else mask
         a = _lib.FtaArgs()
         self.out = torch.full((bsz, hq, L, D), float("nan"), dtype=q.dtype)
-        self.keep = (q, k, v, x["current_k"], x["current_v"], mask, x["kv_seq_len"], tables)
+        lens = x["kv_seq_len"].int() if len32 else x["kv_seq_len"]
+        self.keep = (q, k, v, x["current_k"], x["current_v"], mask, lens, tables)
         a.q, a.k_cache, a.v_cache, a.cur_k, a.cur_v = q.data_ptr(), k.data_ptr(), v.data_ptr(), x["current_k"].data_ptr(), x["current_v"].data_ptr()
-        a.mask, a.kv_seq_len, a.out = mask.data_ptr(), x["kv_seq_len"].data_ptr(), self.out.data_ptr()
+        a.mask, a.kv_seq_len, a.out = mask.data_ptr(), lens.data_ptr(), self.out.data_ptr()
         a.bsz, a.num_q_heads, a.num_kv_heads, a.cur_heads, a.q_len, a.head_dim = bsz, hq, k.size(1), x["current_k"].size(1), L, D
         if tables is not None:
             a.page_size = k.size(2)
@@ -92,7 +94,7 @@ class HostCall:
             a.block_table, a.block_table_stride = tables.data_ptr(), tables.stride(0)
         else:
             a.cache_len = a.v_cache_len = k.size(2)
-        a.block_size, a.max_seq_len_hint, a.dtype, a.len_dtype = 64, hint, DTYPES[q.dtype], _lib.FTA_I64
+        a.block_size, a.max_seq_len_hint, a.dtype, a.len_dtype = block_size, hint, DTYPES[q.dtype], _lib.FTA_I32 if len32 else _lib.FTA_I64
         a.force_splits, a.force_kernel, a.sm_scale = splits, kernel, 1.0 / math.sqrt(D)
         for name, t in (("q_stride", q), ("k_stride", k), ("v_stride", v), ("ck_stride", x["current_k"]), ("cv_stride", x["current_v"]), ("out_stride", self.out)):
             getattr(a, name)[:] = t.stride()[:3]
