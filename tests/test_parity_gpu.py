@@ -305,12 +305,13 @@ def test_lengths_beyond_cache_are_clamped_and_padding_is_ignored():
     check(run(x), ref, torch.bfloat16)
 
 
-@pytest.mark.parametrize("bsz,splits", [(37, 1), (37, 3), (37, 4), (64, 8), (300, 2)])
+@pytest.mark.parametrize("bsz,splits", [(37, 1), (37, 3), (37, 4), (64, 8), (65, 3), (200, 2), (300, 2)])
 def test_ragged_batch_dispatch_order(bsz, splits):
     """Stage 1 resolves its workgroups longest-first from the batch's lengths; every
     (sequence, split) must still be computed exactly once whatever the order: ties, empty
-    caches, lengths that are exact multiples of the chunk, and batches beyond the limit
-    of the ordered dispatch (identity order)."""
+    caches, lengths that are exact multiples of the chunk; batches a wave orders by itself
+    (up to 64), batches ordered through LDS (65 .. 256) and batches beyond the limit of the
+    ordered dispatch (identity order)."""
     g = torch.Generator().manual_seed(bsz * 31 + splits)
     tmax = 512
     lens = torch.randint(0, tmax + 1, (bsz,), generator=g).tolist()
