@@ -2,7 +2,8 @@
 
 The reference's own generator (flash_tree_attn.py:403-414) draws an unseeded random
 {1, -inf} matrix that is not a tree; real callers (Medusa / EAGLE style drafts) hold
-a parent array. These helpers turn a parent array into the ADDITIVE mask the op
+a parent array, or a list of paths from which one follows (`parents_from_paths`). These
+helpers turn a parent array into the ADDITIVE mask the op
 consumes (flash_tree_attn.py:368): 0 where column j is an ancestor of, or equal to,
 row i, and -inf elsewhere; or into the PACKED form, one bit per (row, tree key) in
 64-bit words (8 bytes per row and 64 keys instead of 256), which the kernels expand to
@@ -27,6 +28,52 @@ def random_tree_parents(q_len: int, generator: Optional[torch.Generator] = None)
 def chain_parents(q_len: int) -> torch.Tensor:
     """A chain: token i's parent is i-1; its ancestor mask is the causal mask."""
     return torch.arange(-1, q_len - 1, dtype=torch.int64)
+
+
+def parents_from_paths(paths: Sequence[Sequence[int]]) -> torch.Tensor:
+    """Parent array of a draft tree given the way Medusa-style drafts describe it: one entry per
+    non-root node, the tuple of child ranks that leads to it from the root ((0,), (0, 0), (1,),
+    (0, 1), ...). Node 0 is the root (the last accepted token); the other nodes follow in order of
+    (depth, path), so parents precede their children and siblings are ordered by rank. Every
+    proper prefix of a path must be a path of the list itself."""
+    nodes = sorted({tuple(int(c) for c in path) for path in paths}, key=lambda path: (len(path), path))
+    if any(len(path) == 0 for path in nodes):
+        raise ValueError("the empty path is the root and is not listed")
+    index = {(): 0}
+    parents = [-1]
+    for path in nodes:
+        if path[:-1] not in index:
+            raise ValueError(f"path {list(path)} has no parent {list(path[:-1])} in the list")
+        index[path] = len(parents)
+        parents.append(index[path[:-1]])
+    return torch.tensor(parents, dtype=torch.int64)
+
+
+def path_to_node(parents: Sequence[int], node: int) -> list:
+    """Tree positions from the root to `node`, both included: the accepted path whose K/V rows
+    `append_accepted_kv` moves into the cache once verification has picked `node`."""
+    p = [int(x) for x in parents]
+    if not 0 <= int(node) < len(p):
+        raise ValueError(f"node {node} is not in [0, {len(p)})")
+    path, j = [], int(node)
+    while j >= 0:
+        if len(path) > len(p):
+            raise ValueError("the parent array has a cycle")
+        path.append(j)
+        j = p[j]
+    return path[::-1]
+
+
+def accepted_paths(parents: Sequence[int], nodes: Sequence[int], device=None):
+    """(accept_idx int32 [bsz, longest path], accept_len int64 [bsz]) for `append_accepted_kv`: row b
+    holds the positions from the root to nodes[b], padded with zeros behind accept_len[b]."""
+    paths = [path_to_node(parents, n) for n in nodes]
+    width = max(len(path) for path in paths)
+    idx = torch.zeros(len(paths), width, dtype=torch.int32)
+    for b, path in enumerate(paths):
+        idx[b, : len(path)] = torch.tensor(path, dtype=torch.int32)
+    lens = torch.tensor([len(path) for path in paths], dtype=torch.int64)
+    return (idx.to(device), lens.to(device)) if device is not None else (idx, lens)
 
 
 def ancestor_matrix(parents: Sequence[int]) -> torch.Tensor:
