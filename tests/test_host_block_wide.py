@@ -144,7 +144,7 @@ def test_64_row_wave_kernel_on_host_threads(host_lib, case):
 # Keys of more spread than N(0, 1): a few keys carry each row. The loop's lazy softmax exponentiates against a stale
 # reference, so every probability of a row, its largest included, is rounded to bf16 (2^-9 relative) where the other
 # loops hold the largest exactly at 1, and full tiles take no compensating product with the rounding residue (the
-# 8-wave, 4-wave and key-halves loops do: tests/test_host_block_mfma.py). At twice the spread the loop stays inside
+# 8-wave, 4-wave and key-halves loops do: tests/test_host_block_mfma_forms.py). At twice the spread the loop stays inside
 # the tolerance; at four times it does not (1.06 - 1.42 of atol 2e-3 / rtol 1e-2 here, 3 of 32768 values beyond it
 # on the GPU at 1024 keys). That is a known limit of this opt-in loop: the rows stay here, marked, until it is lifted.
 @pytest.mark.parametrize("scale_k,seed,keys", [

@@ -228,7 +228,7 @@ unproven_on_gpu = pytest.mark.skipif(os.environ.get("FTA_GPU_TESTS_OF_UNPROVEN_K
                                      reason="kernel form not yet run on a GPU as built; set FTA_GPU_TESTS_OF_UNPROVEN_KERNELS=1 to run it")
 # bf16, keys of four times the spread: the lazy softmax of the 64-row-wave loop rounds every probability of a row,
 # its largest included, to bf16 against a stale reference, and carries no compensating product for full tiles: on
-# host threads 1.06 - 1.42 of the tolerance (the other loops: <= 0.4, tests/test_host_block_mfma.py). A known limit
+# host threads 1.06 - 1.42 of the tolerance (the other loops: <= 0.4, tests/test_host_block_mfma_forms.py). A known limit
 # of that opt-in loop, kept visible here.
 wide_loop_peaked_limit = pytest.mark.skip(reason="known limit of the opt-in 64-row-wave loop: bf16 probabilities of peaked rows exceed atol 2e-3 / rtol 1e-2")
 
