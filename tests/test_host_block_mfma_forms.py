@@ -103,3 +103,14 @@ def test_peaked_logits_other_loops(host_lib, form, scale_k, seed):
     assert call.plan.rows_per_wg == rows and call.plan.mfma_loop == loop
     share, bad = share_of_tolerance(call.run(), oracle(x))
     assert bad == 0 and share <= (1.0 if scale_k > 2 else 0.5), (share, bad)
+
+
+def test_one_unit_of_the_headline_workload(host_lib):
+    """One cache head of one sequence of the headline workload (4 query heads x 64 tree tokens = 256 rows, 8192 cached
+    keys, bf16), cut as the plan cuts the whole workload on 256 CUs: 4 splits of 2112 keys, 33 tiles through the fused
+    loop per workgroup, the tree tile on the last. Well inside the tolerance on N(0, 1) data."""
+    x = make(0, 1, 4, 1, 64, 128, 8192, torch.bfloat16, [8192])
+    call = HostCall(host_lib, x, splits=4, kernel=MFMA)
+    assert (call.plan.num_splits, call.plan.chunk, call.plan.rows_per_wg, call.plan.mfma_loop) == (4, 2112, 256, 0)
+    share, bad = share_of_tolerance(call.run(), oracle(x))
+    assert bad == 0 and share <= 0.25, share
