@@ -132,6 +132,7 @@ def oracle(x):
     (3, 4, 2, 3, 32, 2048, torch.bfloat16, [130, 0, 64], 0),          # a cache far larger than the sequences; an empty cache
     (1, 2, 2, 9, 64, 200, torch.float16, [200], 1),                   # one split: straight to `out`, no scratch
     (2, 2, 1, 4, 32, 256, torch.float32, [999, -3], 3),               # a length beyond the cache is clamped, a negative one is empty
+    (70, 1, 1, 2, 32, 192, torch.float32, [(53 * i) % 193 for i in range(70)], 2),   # more than 64 sequences: the ordering pass through LDS, both stages
 ])
 def test_whole_call_on_host_threads(host_lib, shape):
     bsz, hq, hkv, L, D, tmax, dtype, lens, splits = shape
