@@ -53,7 +53,9 @@ typedef enum fta_kernel {
   FTA_KERNEL_MFMA = 1,     /* MFMA tiles: f16/bf16, head_dim 64/128/256, sm_scale > 0; any number of rows */
   FTA_KERNEL_MFMA_WIDE = 2,/* only as fta_args.force_kernel: the MFMA kernel with 64 query rows per wave and the
                               hand-scheduled half-tile loop, for units of more than 128 rows on contiguous caches,
-                              head_dim 64/128. A plan reports it as FTA_KERNEL_MFMA with mfma_loop = 1. */
+                              head_dim 64/128. A plan reports it as FTA_KERNEL_MFMA with mfma_loop = 1. Not the library's
+                              choice anywhere: slower than the default loop where it was timed, and bf16 rows that a few
+                              keys carry can leave atol 2e-3 / rtol 1e-2 in it (the other loops compensate for that). */
   FTA_KERNEL_MFMA_SPLIT_KEYS = 3 /* only as fta_args.force_kernel: the MFMA kernel for units of at most 64 query rows,
                               head_dim 64/128, with two waves per 32-row block that each take half of a tile's keys
                               (all four waves of a workgroup compute). A plan reports it as FTA_KERNEL_MFMA with
